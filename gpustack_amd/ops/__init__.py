@@ -126,6 +126,9 @@ def reshape_and_cache(k, v, k_cache, v_cache, slots) -> None:
 
 
 def greedy_sample_into(out, logits) -> None:
+    if logits.is_cuda and logits.dtype == torch.float32:
+        _load_latent().argmax_f32(out, logits)  # fp32-logit models
+        return
     hip = _backend(logits)
     if hip is not None:
         hip.greedy_sample(out, logits)
@@ -135,6 +138,9 @@ def greedy_sample_into(out, logits) -> None:
 
 def greedy_sample(logits) -> torch.Tensor:
     out = torch.empty(logits.shape[0], dtype=torch.long, device=logits.device)
+    if logits.is_cuda and logits.dtype == torch.float32:
+        _load_latent().argmax_f32(out, logits)  # fp32-logit models
+        return out
     hip = _backend(logits)
     if hip is not None:
         hip.greedy_sample(out, logits)
@@ -342,3 +348,185 @@ def mfma_probe(a, b):
 
 
 build_cos_sin_cache = torch_ref.build_cos_sin_cache
+
+
+# --- fp32-residual op family ------------------------------------------------
+# Kernels for models that keep the residual stream, norms, attention scores
+# and routers in fp32 (ModelSpec.fp32_residual): ops/csrc/resid32.hip and
+# ops/csrc/latent_attn.hip, built into their own small extension so a
+# checkout that serves only such a model compiles nothing else. Activations
+# entering GEMMs are bf16 or fp32 (the engine dtype); every kernel is
+# instantiated for both.
+
+_LATENT = None
+
+
+def _load_latent():
+    """Load `_hip_latent.so`, compiling it in-tree first when no built
+    library is there (a fresh checkout on a GPU box)."""
+    global _LATENT
+    if _LATENT is not None:
+        return _LATENT
+    import importlib.util
+
+    from .build import LATENT_SO_PATH, build_latent
+
+    if not LATENT_SO_PATH.exists():
+        build_latent()
+    spec = importlib.util.spec_from_file_location(
+        "gpustack_amd.ops._hip_latent", LATENT_SO_PATH)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    _LATENT = mod
+    return mod
+
+
+def _lat_backend(t: torch.Tensor):
+    return _load_latent() if t.is_cuda else None
+
+
+ACT_MODES = {"relu2": 0, "gelu": 1, "gelu_tanh": 2, "silu": 3}
+
+
+def embed_pair_hash(x, h, tokens, prev, embed, pair_table, buckets: int,
+                    mul_prev: int, mul_cur: int) -> None:
+    k = _lat_backend(x)
+    if k is not None:
+        k.embed_pair_hash(x, h, tokens, prev, embed, pair_table,
+                          buckets, mul_prev, mul_cur)
+    else:
+        torch_ref.embed_pair_hash(x, h, tokens, prev, embed, pair_table,
+                                  buckets, mul_prev, mul_cur)
+
+
+def rms_scale_add(x, a, weight, scale, eps: float, h) -> None:
+    k = _lat_backend(x)
+    if k is not None:
+        k.rms_scale_add(x, a, weight, scale, eps, h)
+    else:
+        torch_ref.rms_scale_add(x, a, weight, scale, eps, h)
+
+
+def rms_norm_f32(out, x, weight, eps: float) -> None:
+    k = _lat_backend(x)
+    if k is not None:
+        k.rms_norm_f32(out, x, weight, eps)
+    else:
+        torch_ref.rms_norm_f32(out, x, weight, eps)
+
+
+def latent_norm_store(cache, src, col0: int, weight, slots, eps: float) -> None:
+    k = _lat_backend(src)
+    if k is not None:
+        k.latent_norm_store(cache, src, col0, weight, slots, eps)
+    else:
+        torch_ref.latent_norm_store(cache, src, col0, weight, slots, eps)
+
+
+_LAT_GROUP = 16   # (row, head) pairs sharing one key stream per workgroup
+
+
+def build_latent_tiles(seq_starts, seq_hists, seq_news, heads: int, device):
+    """Group the batch's (row, head) pairs into tiles of at most 16 pairs
+    that belong to ONE sequence, so a workgroup streams that sequence's
+    latents once for all of them. Long portions tile as 16 rows x 1 head;
+    short ones (decode rows above all) pack rows x heads. Returns int32
+    [ntiles, 6]: row0, nrows, head0, nheads, seq, pos0."""
+    tiles = []
+    G = _LAT_GROUP
+    for i, (st, hist, new) in enumerate(zip(seq_starts, seq_hists, seq_news)):
+        if new >= G:
+            nh, nr = 1, G
+        else:
+            nh = min(heads, G)
+            nr = max(1, min(new, G // nh))
+        for r0 in range(0, new, nr):
+            n = min(nr, new - r0)
+            for h0 in range(0, heads, nh):
+                tiles.append((st + r0, n, h0, min(nh, heads - h0), i,
+                              hist + r0))
+    return torch.tensor(tiles, dtype=torch.int32, device=device).view(-1, 6)
+
+
+def latent_attention_mfma_ok(cache) -> bool:
+    """True when ops.latent_attention takes the MFMA kernel for this pool:
+    bf16, both page planes, 16-token pages, width % 32 == 0 (<= 1024). Only
+    then may q_lat / ctx be bf16 and arbitrarily strided."""
+    return (cache.is_cuda and cache.dtype == torch.bfloat16
+            and cache.shape[1] == 2 and cache.shape[2] == 16
+            and cache.shape[3] % 32 == 0 and cache.shape[3] <= 1024)
+
+
+def latent_attention(ctx, q_lat, cache, block_tables, row_seq, positions,
+                     scale: float, tiles=None, exact: bool = False,
+                     max_ctx: int = 0) -> None:
+    """ctx / q_lat: [T, H, R] views (last axis contiguous). `exact` forces
+    the fp32 vector-ALU kernel where the MFMA kernel would run. `max_ctx`
+    (longest context in the batch, a host number) lets a batch of few tiles
+    over long contexts split each tile's keys over several workgroups."""
+    k = _lat_backend(q_lat)
+    if k is not None:
+        if tiles is None:
+            raise ValueError("latent_attention on GPU needs the tile list "
+                             "(build_latent_tiles)")
+        nsplit = 1
+        nt = tiles.shape[0]
+        if not exact and max_ctx >= 512 and 0 < nt < 512:
+            nsplit = max(1, min(16, 1024 // nt, max_ctx // 128))
+        k.latent_attention(ctx, q_lat, cache, block_tables, tiles, positions,
+                           scale, exact, nsplit)
+    else:
+        torch_ref.latent_attention(ctx, q_lat, cache, block_tables, row_seq,
+                                   positions, scale)
+
+
+def act_inplace(x, mode: str) -> None:
+    k = _lat_backend(x)
+    if k is not None:
+        k.act_inplace(x, ACT_MODES[mode])
+    else:
+        torch_ref.act_inplace(x, mode)
+
+
+def route_grouped_topk(experts, weights, logits, n_experts: int, groups: int,
+                       keep: int, scale: float) -> None:
+    k = _lat_backend(logits)
+    if k is not None:
+        k.route_grouped_topk(experts, weights, logits, n_experts, groups,
+                             keep, scale)
+    else:
+        torch_ref.route_grouped_topk(experts, weights, logits, n_experts,
+                                     groups, keep, scale)
+
+
+def moe_combine(out, y, inv, weights, shared, gate_logits, gate_col: int) -> None:
+    k = _lat_backend(out)
+    if k is not None:
+        k.moe_combine(out, y, inv, weights, shared, gate_logits, gate_col)
+    else:
+        torch_ref.moe_combine(out, y, inv, weights, shared, gate_logits,
+                              gate_col)
+
+
+def grouped_ff_available(x, width: int, ff: int) -> bool:
+    """The sync-free grouped expert kernels take bf16 on the GPU with
+    width % 64 == 0 and ff % 64 == 0."""
+    return (x.is_cuda and x.dtype == torch.bfloat16
+            and width % 64 == 0 and ff % 64 == 0)
+
+
+def grouped_up_act(u, x, up_w, s_tok, offs, counts, mode: str) -> None:
+    _load_latent().grouped_up_act(u, x, up_w, s_tok, offs, counts,
+                                  ACT_MODES[mode])
+
+
+def grouped_down(y, u, down_w, offs, counts) -> None:
+    _load_latent().grouped_down(y, u, down_w, offs, counts)
+
+
+def softcap_(logits, cap: float) -> None:
+    k = _lat_backend(logits)
+    if k is not None:
+        k.softcap(logits, cap)
+    else:
+        torch_ref.softcap_(logits, cap)

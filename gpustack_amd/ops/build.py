@@ -20,6 +20,11 @@ ARCH = os.environ.get("GPUSTACK_AMD_ARCH", "gfx950")
 
 HIP_SOURCES = ["pointwise.hip", "attn_decode.hip", "attn_prefill.hip", "skinny_gemm.hip", "gemm8.hip", "gemm8_lab.hip", "moe_gemm.hip", "w4_gemm.hip", "mla_decode.hip"]
 CPP_SOURCES = ["bindings.cpp"]
+# the fp32-residual op family lives in its own small library: a checkout
+# that serves only such a model compiles these few files and nothing else
+LATENT_SO_PATH = PKG_DIR / "_hip_latent.so"
+LATENT_SOURCES = ["resid32.hip", "latent_attn.hip", "grouped_ff.hip",
+                  "latent_bindings.cpp"]
 
 
 def _torch_paths():
@@ -37,9 +42,11 @@ def _torch_paths():
     return includes, libdir, abi
 
 
-def _common_flags(abi: str):
+def _common_flags(abi: str, ext_name: str = "_hip_ops"):
     return [
         "-O3",
+        # no packed-fp32 VALU forms (v_pk_*_f32) from ordinary float code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         "-std=c++17",
         "-fPIC",
         f"--offload-arch={ARCH}",
@@ -48,7 +55,7 @@ def _common_flags(abi: str):
         "-D__HIP_PLATFORM_AMD__=1",
         "-DHIPBLAS_V2",
         "-DHIP_ENABLE_WARP_SYNC_BUILTINS=1",
-        "-DTORCH_EXTENSION_NAME=_hip_ops",
+        f"-DTORCH_EXTENSION_NAME={ext_name}",
         "-Wno-unused-result",
         "-fvisibility=hidden",
     ]
@@ -122,6 +129,52 @@ def build(verbose: bool = False, force: bool = False) -> Path:
     return SO_PATH
 
 
+def build_latent(verbose: bool = False, force: bool = True) -> Path:
+    """Compile the fp32-residual op family into `_hip_latent.so`. Objects
+    are built under a private name and the library is moved into place at
+    the end, so a concurrent reader never sees a half-written file."""
+    includes, libdir, abi = _torch_paths()
+    inc_flags = [f"-I{p}" for p in includes]
+    flags = _common_flags(abi, "_hip_latent")
+    build_dir = CSRC / ".build_latent"
+    build_dir.mkdir(exist_ok=True)
+    newest = max((CSRC / s).stat().st_mtime
+                 for s in LATENT_SOURCES + ["common.h"])
+    if (LATENT_SO_PATH.exists() and not force
+            and LATENT_SO_PATH.stat().st_mtime >= newest):
+        return LATENT_SO_PATH
+    cmds, objs = [], []
+    for src in LATENT_SOURCES:
+        obj = build_dir / (Path(src).stem + ".o")
+        cmd = ["hipcc", *flags, *inc_flags, "-c", str(CSRC / src), "-o", str(obj)]
+        if src.endswith(".cpp"):
+            cmd[1:1] = ["-x", "hip"]
+        cmds.append(cmd)
+        objs.append(str(obj))
+    if verbose:
+        for c in cmds:
+            print(" ".join(c), file=sys.stderr)
+    procs = [subprocess.Popen(c, stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                              text=True) for c in cmds]
+    for c, pr in zip(cmds, procs):
+        _out, err = pr.communicate()
+        if pr.returncode != 0:
+            raise RuntimeError(f"build command failed ({' '.join(c[:3])} ...):"
+                               f"\n{err[-8000:]}")
+    tmp = build_dir / f"_hip_latent.{os.getpid()}.so"
+    _run(["hipcc", "-shared", f"--offload-arch={ARCH}", *objs, f"-L{libdir}",
+          "-ltorch", "-ltorch_hip", "-ltorch_cpu", "-lc10", "-lc10_hip",
+          "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
+          f"-Wl,-rpath,{libdir}", "-o", str(tmp)])
+    os.replace(tmp, LATENT_SO_PATH)
+    return LATENT_SO_PATH
+
+
 if __name__ == "__main__":
-    build(verbose=True, force="--force" in sys.argv)
-    print(f"built {SO_PATH}")
+    if "--latent" in sys.argv:
+        build_latent(verbose=True)
+        print(f"built {LATENT_SO_PATH}")
+    else:
+        build(verbose=True, force="--force" in sys.argv)
+        build_latent(verbose=True)
+        print(f"built {SO_PATH} {LATENT_SO_PATH}")

@@ -320,3 +320,138 @@ def paged_prefill_attn(
         att = _sink_softmax(att, sinks)
         out[start:start + new] = (att @ vals).permute(1, 0, 2).to(out.dtype)
         row += new
+
+
+# --- fp32-residual op family (heterogeneous latent-attention stacks) -------
+# The residual stream is fp32; GEMM operands take the model dtype. These are
+# the CPU execution path and the numerics oracle of ops/csrc/resid32.hip and
+# ops/csrc/latent_attn.hip.
+
+def embed_pair_hash(x: torch.Tensor, h: torch.Tensor | None,
+                    tokens: torch.Tensor, prev: torch.Tensor,
+                    embed: torch.Tensor, pair_table: torch.Tensor | None,
+                    buckets: int, mul_prev: int, mul_cur: int) -> None:
+    """x[t] = embed[tok] + pair_table[(prev*mul_prev + tok*mul_cur) %
+    buckets] in fp32; prev < 0 marks a sequence's first token, which reads
+    row `buckets`. h (optional) receives x rounded to the GEMM dtype."""
+    v = embed[tokens].float()
+    if pair_table is not None:
+        row = (prev * mul_prev + tokens * mul_cur) % buckets
+        row = torch.where(prev < 0, torch.full_like(row, buckets), row)
+        v = v + pair_table[row].float()
+    x.copy_(v)
+    if h is not None:
+        h.copy_(v.to(h.dtype))
+
+
+def rms_scale_add(x: torch.Tensor, a: torch.Tensor, weight: torch.Tensor,
+                  scale: torch.Tensor | None, eps: float,
+                  h: torch.Tensor | None) -> None:
+    """x += a / sqrt(mean(a^2) + eps) * weight [* scale], all in fp32 on the
+    fp32 stream x; h (optional) receives the new x in the GEMM dtype."""
+    af = a.float()
+    y = af * torch.rsqrt(af.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    if scale is not None:
+        y = y * scale.float()
+    x.add_(y)
+    if h is not None:
+        h.copy_(x.to(h.dtype))
+
+
+def rms_norm_f32(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor,
+                 eps: float) -> None:
+    xf = x.float()
+    out.copy_((xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+               * weight.float()).to(out.dtype))
+
+
+def latent_norm_store(cache: torch.Tensor, src: torch.Tensor, col0: int,
+                      weight: torch.Tensor, slots: torch.Tensor,
+                      eps: float) -> None:
+    """RMS-normalise src[:, col0:col0+R] in fp32 and write each row into
+    its slot of the paged latent pool [nblocks, P, BS, R] (slot < 0: skip):
+    plane 0 row-major, plane 1 (if present) the page transposed [R][BS]."""
+    nb, P, BS, R = cache.shape
+    lat = src[:, col0:col0 + R].float()
+    c = (lat * torch.rsqrt(lat.pow(2).mean(-1, keepdim=True) + eps)
+         * weight.float()).to(cache.dtype)
+    ok = slots >= 0
+    blk, off = slots[ok] // BS, slots[ok] % BS
+    cache[blk, 0, off] = c[ok]
+    if P == 2:
+        tr = cache.view(nb, P, BS * R)[:, 1].unflatten(-1, (R, BS))
+        tr[blk, :, off] = c[ok]
+
+
+def latent_attention(ctx: torch.Tensor, q_lat: torch.Tensor,
+                     cache: torch.Tensor, block_tables: torch.Tensor,
+                     row_seq: torch.Tensor, positions: torch.Tensor,
+                     scale: float) -> None:
+    """ctx[t, h] = softmax_j<=pos(t)(q_lat[t, h] . c_j * scale) . C for the
+    latents c_j of row t's sequence, read through its block table."""
+    T, H, R = q_lat.shape
+    BS = cache.shape[2]
+    for t in range(T):
+        L = int(positions[t]) + 1
+        bt = block_tables[int(row_seq[t])]
+        j = torch.arange(L, device=cache.device)
+        C = cache[bt[j // BS].long(), 0, j % BS].float()     # [L, R]
+        s = (q_lat[t].float() @ C.T) * scale                 # [H, L]
+        p = torch.softmax(s, dim=-1)
+        ctx[t] = p @ C
+
+
+def act_inplace(x: torch.Tensor, mode: str) -> None:
+    xf = x.float()
+    if mode == "relu2":
+        y = torch.relu(xf) ** 2
+    elif mode == "gelu":
+        y = torch.nn.functional.gelu(xf)
+    elif mode == "gelu_tanh":
+        y = torch.nn.functional.gelu(xf, approximate="tanh")
+    elif mode == "silu":
+        y = torch.nn.functional.silu(xf)
+    else:
+        raise ValueError(mode)
+    x.copy_(y.to(x.dtype))
+
+
+def route_grouped_topk(experts: torch.Tensor, weights: torch.Tensor,
+                       logits: torch.Tensor, n_experts: int, groups: int,
+                       keep: int, scale: float) -> None:
+    """Softmax over logits[:, :n_experts]; experts outside the `keep`
+    groups with the largest best-member score are masked; the top-k of the
+    rest are written with weight score * scale."""
+    T = logits.shape[0]
+    top = experts.shape[1]
+    s = torch.softmax(logits[:, :n_experts].float(), dim=-1)
+    choice = s
+    if groups > 1 and keep < groups:
+        g = s.view(T, groups, n_experts // groups).amax(-1)
+        gi = torch.topk(g, keep, dim=-1)[1]
+        gm = torch.zeros_like(g, dtype=torch.bool).scatter_(1, gi, True)
+        em = gm.unsqueeze(-1).expand(T, groups, n_experts // groups)
+        choice = s.masked_fill(~em.reshape(T, n_experts), -1.0)
+    idx = torch.topk(choice, top, dim=-1)[1]
+    experts.copy_(idx.to(experts.dtype))
+    weights.copy_(s.gather(1, idx) * scale)
+
+
+def moe_combine(out: torch.Tensor, y: torch.Tensor, inv: torch.Tensor,
+                weights: torch.Tensor, shared: torch.Tensor | None,
+                gate_logits: torch.Tensor | None, gate_col: int) -> None:
+    """out[t] = sum_k weights[t, k] * y[inv[t, k]] (+ sigmoid(gate) *
+    shared[t]) in fp32."""
+    T, top = inv.shape
+    acc = (y[inv.reshape(-1).long()].float().view(T, top, -1)
+           * weights.unsqueeze(-1)).sum(1)
+    if shared is not None:
+        sh = shared.float()
+        if gate_logits is not None:
+            sh = sh * torch.sigmoid(gate_logits[:, gate_col:gate_col + 1].float())
+        acc = acc + sh
+    out.copy_(acc)
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> None:
+    logits.copy_(cap * torch.tanh(logits / cap))
