@@ -11,6 +11,46 @@ from dataclasses import dataclass, field
 from pathlib import Path
 
 
+@dataclass(frozen=True)
+class LatentMixerSpec:
+    """Position-free latent attention (models/latent_attention.py): keys
+    and values of every head are linear images of ONE normalised latent of
+    width kv_rank per token, which is all the paged cache holds."""
+    heads: int
+    qk_dim: int
+    v_dim: int
+    kv_rank: int
+    scale: float
+
+
+@dataclass(frozen=True)
+class FeedForwardSpec:
+    """Ungated feed-forward W_down act(W_up h), dense or as a bank of
+    routed experts (models/experts.py). Routing: softmax scores over all
+    experts, group-limited top-k (groups of neighbouring experts ranked by
+    their best member, keep_groups stay eligible), weights = score *
+    route_scale without renormalisation; shared_ff > 0 adds an always-on
+    expert scaled by a per-token sigmoid gate when shared_gated."""
+    kind: str = "dense"                  # "dense" | "moe"
+    ff: int = 0                          # dense width / routed expert width
+    act: str = "relu2"                   # "relu2" | "gelu" | "gelu_tanh" | "silu"
+    experts: int = 0
+    top: int = 0
+    groups: int = 1
+    keep_groups: int = 1
+    route_scale: float = 1.0
+    shared_ff: int = 0
+    shared_gated: bool = False
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    """One entry of a heterogeneous layer stack (ModelSpec.layers)."""
+    mixer_type: str
+    mixer: LatentMixerSpec
+    mlp: FeedForwardSpec | None = None
+
+
 @dataclass
 class ModelSpec:
     architecture: str = "LlamaForCausalLM"
@@ -112,12 +152,29 @@ class ModelSpec:
     parallel_block: bool = False         # Cohere: x + attn(ln(x)) + mlp(ln(x))
     logits_multiplier: float = 0.0       # Cohere logit_scale (multiplies)
     mlp_no_gate: bool = False            # Arcee: down(act(up(x))), no gate
+    # Heterogeneous stacks (Vunitar): one LayerSpec per layer — each layer
+    # names its mixer and feed-forward with their own sizes, so nothing
+    # above (num_heads, head_dim, intermediate_size, ...) describes them.
+    # Such models keep the residual stream, norms, scores and routers in
+    # fp32 (fp32_residual) and run norm-after layers with a learned
+    # per-channel layer scale on each sublayer's normed output.
+    layers: tuple | None = None
+    fp32_residual: bool = False
+    layer_scale: bool = False
+    # hashed (previous token, token) embedding added to the token row:
+    # row = (prev * mul_prev + tok * mul_cur) % buckets; a sequence's first
+    # token reads the extra row `buckets`. 0 buckets = off
+    bigram_buckets: int = 0
+    bigram_mul_prev: int = 0
+    bigram_mul_cur: int = 0
 
     @property
     def gqa_ratio(self) -> int:
         return self.num_heads // self.num_kv_heads
 
     def kv_bytes_per_token(self, dtype_size: int = 2) -> int:
+        if self.layers is not None:
+            return sum(ls.mixer.kv_rank for ls in self.layers) * dtype_size
         if self.kv_lora_rank:
             # MLA: one compressed latent row per token per layer
             return (self.num_layers
@@ -127,6 +184,26 @@ class ModelSpec:
 
     def weight_bytes(self, dtype_size: int = 2) -> int:
         h, i, v = self.hidden_size, self.intermediate_size, self.vocab_size
+        if self.layers is not None:
+            n = 2 * v * h + h
+            if self.bigram_buckets:
+                n += (self.bigram_buckets + 1) * h
+            for ls in self.layers:
+                m = ls.mixer
+                n += (h * m.heads * m.qk_dim + h * m.kv_rank + m.kv_rank
+                      + m.kv_rank * m.heads * (m.qk_dim + m.v_dim)
+                      + m.heads * m.v_dim * h + 2 * h)
+                f = ls.mlp
+                if f is None:
+                    continue
+                n += 2 * h
+                if f.kind == "moe":
+                    n += f.experts * (2 * h * f.ff + h)
+                    if f.shared_ff:
+                        n += 2 * h * f.shared_ff + h
+                else:
+                    n += 2 * h * f.ff
+            return n * dtype_size
         if self.kv_lora_rank:
             dq = self.qk_nope_head_dim + self.qk_rope_head_dim
             qp = (self.q_lora_rank * (h + self.num_heads * dq)
@@ -170,7 +247,68 @@ class ModelSpec:
         return sc
 
     @classmethod
+    def _from_vunitar_config(cls, cfg: dict) -> "ModelSpec":
+        """Vunitar checkpoints describe themselves layer by layer: `layers`
+        is a list of {type, mixer{...}, mlp{...}|null}; every size and
+        every per-model constant comes from there."""
+        layers = []
+        for ent in cfg["layers"]:
+            if ent["type"] != "latent_attention":
+                raise NotImplementedError(
+                    f"Vunitar mixer type {ent['type']!r} is not implemented")
+            m = ent["mixer"]
+            mixer = LatentMixerSpec(
+                heads=int(m["heads"]), qk_dim=int(m["dim"]),
+                v_dim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
+                scale=float(m["scale"]))
+            f = ent.get("mlp")
+            if not f:
+                ff = None
+            elif f["kind"] == "dense":
+                ff = FeedForwardSpec(kind="dense", ff=int(f["ff"]),
+                                     act="relu2")
+            elif f["kind"] == "moe":
+                r = f["router"]
+                g = r.get("groups") or {}
+                sh = f.get("shared") or None
+                ff = FeedForwardSpec(
+                    kind="moe", ff=int(f["expert"]["ff"]), act="gelu",
+                    experts=int(r["experts"]), top=int(r["top"]),
+                    groups=int(g.get("count", 1) or 1),
+                    keep_groups=int(g.get("keep", g.get("count", 1)) or 1),
+                    route_scale=float(r.get("scale", 1.0)),
+                    shared_ff=int(sh["ff"]) if sh else 0,
+                    shared_gated=bool(sh))
+            else:
+                raise NotImplementedError(
+                    f"Vunitar feed-forward kind {f['kind']!r}")
+            layers.append(LayerSpec("latent_attention", mixer, ff))
+        bg = (cfg.get("embedding") or {}).get("bigram") or {}
+        return cls(
+            architecture="Vunitar",
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            num_layers=len(layers),
+            layers=tuple(layers),
+            # filler for code that sizes things by head: one latent "head"
+            num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+            rms_norm_eps=float(cfg["norm"]["eps"]),
+            # no positional signal anywhere: length is bounded by the
+            # cache pool alone
+            max_position_embeddings=int(
+                cfg.get("max_position_embeddings", 1 << 20)),
+            eos_token_id=int(cfg.get("eos_token_id", -1)),
+            norm_after=True, layer_scale=True, fp32_residual=True,
+            final_logit_softcap=float(cfg.get("logit_softcap") or 0.0),
+            bigram_buckets=int(bg.get("buckets", 0) or 0),
+            bigram_mul_prev=int(bg.get("mul_prev", 0) or 0),
+            bigram_mul_cur=int(bg.get("mul_cur", 0) or 0),
+        )
+
+    @classmethod
     def from_hf_config(cls, cfg: dict) -> "ModelSpec":
+        if cfg.get("architecture") == "Vunitar" and "architectures" not in cfg:
+            return cls._from_vunitar_config(cfg)
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
         if arch.startswith("Cohere") and cfg.get("use_qk_norm"):
             raise NotImplementedError(

@@ -24,6 +24,39 @@ from ..parallel import Communicator
 
 
 @dataclass
+class RaggedMeta:
+    """One uniform description of ANY batch kind (prefill, history
+    continuation, decode, mixed) for models whose mixers read the paged
+    pool row by row: every row belongs to a sequence (row_seq) whose block
+    table is block_tables[row_seq]; a row at position p attends the pool
+    positions 0..p of that sequence. Built by the model runner for models
+    that set `uses_ragged_meta`."""
+
+    block_tables: torch.Tensor    # [nseq, maxb] int32
+    row_seq: torch.Tensor         # [T] int32
+    pos32: torch.Tensor           # [T] int32 copy of positions
+    prev_tokens: torch.Tensor     # [T] int64, -1 = first token of its sequence
+    seq_starts: list              # per seq: first row / tokens already cached /
+    seq_hists: list               # rows in this step
+    seq_news: list
+    max_ctx: int = 0              # longest context (host number)
+    _tiles: dict | None = None
+
+    def latent_tiles(self, heads: int):
+        """Workgroup tile list for ops.latent_attention, cached per head
+        count (layers of one model may differ in it)."""
+        if self._tiles is None:
+            self._tiles = {}
+        t = self._tiles.get(heads)
+        if t is None:
+            t = ops.build_latent_tiles(self.seq_starts, self.seq_hists,
+                                       self.seq_news, heads,
+                                       self.block_tables.device)
+            self._tiles[heads] = t
+        return t
+
+
+@dataclass
 class ForwardMeta:
     """Per-step tensors describing the batch (built by the model runner)."""
 
@@ -55,6 +88,7 @@ class ForwardMeta:
     # sequences (slot_mapping is then the full-batch mapping, positions
     # stay local-row)
     cp: object | None = None
+    ragged: RaggedMeta | None = None
 
 
 class W4Pack:

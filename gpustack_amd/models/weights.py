@@ -48,8 +48,83 @@ def _kv_slice(full, rank: int, tp: int, n_kv: int, d: int):
     return full[head * d:(head + 1) * d]
 
 
+def _layered_tensor_plan(model):
+    """(checkpoint name, destination parameter view, transform) triples for
+    a heterogeneous-stack model (models/vunitar.py). Checkpoint linears are
+    [out, in]; the serving layout fuses q with the latent down-projection,
+    stacks expert banks, keeps the absorbed U_k/U_v factors head-major and
+    the router (+ shared-expert gate row) in fp32."""
+    plan = []
+    same = lambda t: t
+    plan.append(("embed", model.embed, same))
+    if model.pair_table is not None:
+        plan.append(("bigram", model.pair_table, same))
+    plan.append(("final.norm", model.final_norm, same))
+    plan.append(("head", model.lm_head, same))
+    for i, layer in enumerate(model.layers):
+        p = f"l{i}."
+        a = layer.attn
+        nq = a.h * a.dq
+        plan += [
+            (p + "mix.q", a.qd_w[:nq], same),
+            (p + "mix.dkv", a.qd_w[nq:], same),
+            (p + "mix.dkv.norm", a.lat_norm, same),
+            (p + "mix.uk", a.uk, lambda t, a=a: t.view(a.h, a.dq, a.r)),
+            (p + "mix.uv", a.uv_t,
+             lambda t, a=a: t.view(a.h, a.dv, a.r).transpose(1, 2)),
+            (p + "mix.o", a.o_w, same),
+            (p + "norm1", layer.norm1, same),
+            (p + "ls1", layer.ls1, same),
+        ]
+        m = layer.mlp
+        if m is None:
+            continue
+        plan += [(p + "norm2", layer.norm2, same), (p + "ls2", layer.ls2, same)]
+        if hasattr(m, "router_w"):
+            plan.append((p + "mlp.router", m.router_w[:m.e], same))
+            for e in range(m.e):
+                plan.append((p + f"mlp.e{e}.up", m.up_w[e], same))
+                plan.append((p + f"mlp.e{e}.down", m.down_w[e], same))
+            if m.shared_up_w is not None:
+                plan.append((p + "mlp.shared.up", m.shared_up_w, same))
+                plan.append((p + "mlp.shared.down", m.shared_down_w, same))
+                if m.gated:
+                    plan.append((p + "mlp.shared.sg", m.router_w[m.e:], same))
+        else:
+            plan.append((p + "mlp.up", m.up_w, same))
+            plan.append((p + "mlp.down", m.down_w, same))
+    return plan
+
+
+def _random_init_layered(model, cfg: EngineConfig) -> None:
+    """Random weights for a heterogeneous-stack model: projections N(0,
+    1/fan_in), norm and layer-scale weights near 1 / near 0.5, so deep
+    random stacks keep O(1) activations."""
+    for name, dst, fn in _layered_tensor_plan(model):
+        if dst.dim() == 1 and not name.endswith(("router", "sg")):
+            base = 0.5 if name.rsplit(".", 1)[-1] in ("ls1", "ls2") else 1.0
+            t = base + _gen(tuple(dst.shape), name, cfg.seed, torch.float32,
+                            model.device, std=0.05)
+            dst.copy_(t.to(dst.dtype))
+            continue
+        # generate in the checkpoint's own [out, in] shape, then apply the
+        # same layout transform the loader uses
+        if name.endswith("mix.uk"):
+            a_shape = (dst.shape[0] * dst.shape[1], dst.shape[2])
+        elif name.endswith("mix.uv"):
+            a_shape = (dst.shape[0] * dst.shape[2], dst.shape[1])
+        else:
+            a_shape = tuple(dst.shape)
+        fan_in = a_shape[-1]
+        std = 1.0 if name in ("embed", "bigram") else fan_in ** -0.5
+        t = _gen(a_shape, name, cfg.seed, torch.bfloat16, model.device, std=std)
+        dst.copy_(fn(t).to(dst.dtype))
+
+
 def random_init(model, cfg: EngineConfig) -> None:
     spec = model.spec
+    if spec.layers is not None:
+        return _random_init_layered(model, cfg)
     tp, rank = cfg.tp_size, cfg.tp_rank
     dtype, device = model.dtype, model.device
     seed = cfg.seed
@@ -247,6 +322,20 @@ def load_safetensors(model, cfg: EngineConfig, model_dir: str | Path) -> None:
     def get(name):
         t = maybe_dequant(tensors, name, qc)
         return t.to(model.dtype)
+
+    if spec.layers is not None:
+        plan = _layered_tensor_plan(model)
+        missing = [n for n, _, _ in plan if n not in tensors]
+        if missing:
+            raise KeyError(f"checkpoint lacks tensors: {missing[:8]}")
+        for name, dst, fn in plan:
+            t = tensors[name]
+            if tuple(fn(t).shape) != tuple(dst.shape):
+                raise ValueError(
+                    f"{name}: checkpoint shape {tuple(t.shape)} does not fit "
+                    f"the configured {tuple(dst.shape)}")
+            dst.copy_(fn(t).to(dst.dtype))
+        return
 
     pre = "model."
     off = getattr(model, "layer_offset", 0)

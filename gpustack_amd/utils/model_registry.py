@@ -62,7 +62,14 @@ def categories_for_model(source: str, ref: str) -> list[str] | None:
         if cfg.exists():
             try:
                 with open(cfg) as f:
-                    arch = (json.load(f).get("architectures") or [None])[0]
+                    doc = json.load(f)
+                # layer-listed checkpoints name themselves in the singular
+                arch = ((doc.get("architectures") or [None])[0]
+                        or doc.get("architecture"))
+                if arch == "Vunitar" and any(
+                        (ent.get("mlp") or {}).get("kind") == "moe"
+                        for ent in doc.get("layers", [])):
+                    return ["llm", "moe"]
             except (OSError, json.JSONDecodeError):
                 arch = None
     return categories_for_architecture(arch) if arch else None
