@@ -44,6 +44,10 @@ class LLMEngine:
             os.environ.get("GPUSTACK_AMD_ASYNC", "1") == "1"
             and self.comm.world_size == 1
             and cfg.speculative is None
+            # a hashed pair embedding needs the previous token on the host
+            # when the step is assembled; the async pipeline feeds it
+            # device-side one step late
+            and not cfg.spec.bigram_buckets
         )
         self._pending: tuple[list[Sequence], object] | None = None
         self._carry_outputs: list[StepOutput] = []
@@ -355,6 +359,41 @@ class LLMEngine:
         if seq.num_tokens >= self.cfg.max_model_len:
             return "length"
         return None
+
+    # -- forced-token replay ------------------------------------------------
+    def replay_step(self, entries, end=()):
+        """One step of a recorded trace: entries are (request_id, tokens,
+        wanted) — the request's NEXT tokens and the places among them whose
+        logits are returned; `end` lists requests that are finished after
+        the step (their blocks go back to the pool). All entries run as one
+        batch through the scheduler's forced-token path, the model runner
+        and the paged pool of the generation path. Returns fp32 logits
+        [sum(len(wanted)), vocab] in entry order."""
+        if self._pending is not None:
+            self._carry_outputs.extend(self._drain())
+        replay = self.__dict__.setdefault("_replay_seqs", {})
+        plan = []
+        for rid, tokens, wanted in entries:
+            seq = replay.get(rid)
+            if seq is None:
+                if len(replay) >= self.cfg.max_num_seqs:
+                    raise RuntimeError("too many live requests")
+                seq = Sequence(rid, [], SamplingParams(max_tokens=0))
+                replay[rid] = seq
+            seq.prompt_token_ids.extend(int(t) for t in tokens)
+            if seq.num_tokens > self.cfg.max_model_len:
+                raise ValueError("request longer than max_model_len")
+            plan.append((seq, len(tokens), list(wanted)))
+        logits = None
+        if plan:
+            batch = self.scheduler.schedule_forced(plan)
+            logits = self.runner.forward_logits(batch)
+        for rid in end:
+            seq = replay.pop(rid, None)
+            if seq is not None:
+                self.scheduler.release(seq)
+                seq.finish("stop")
+        return logits
 
     # convenience for tests / offline use
     def generate(self, prompts: list[list[int]], params: SamplingParams | None = None):

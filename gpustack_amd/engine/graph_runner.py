@@ -17,7 +17,7 @@ import os
 
 import torch
 
-from ..models.llama import ForwardMeta
+from ..models.llama import ForwardMeta, RaggedMeta
 from .scheduler import ScheduledBatch
 
 BUCKETS = [1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 192, 224, 256,
@@ -73,12 +73,24 @@ class DecodeGraphRunner:
         # persistent — every tensor a captured graph references must outlive
         # the graph (an ephemeral arange here caused replay-time faults)
         self.logits_idx = torch.arange(mb, dtype=torch.long, device=dev)
+        # models that read the pool through the ragged batch view also get
+        # static buffers for it: a decode row is its own one-row sequence
+        # (row i uses block table row i), plus each row's previous token
+        self.ragged = bool(getattr(runner, "ragged", False))
+        if self.ragged:
+            self.prev = torch.full((mb,), -1, dtype=torch.long, device=dev)
+            self.pos32 = torch.zeros(mb, dtype=torch.int32, device=dev)
+            self.row_seq = torch.arange(mb, dtype=torch.int32, device=dev)
+            self.h_prev = torch.full((mb,), -1, dtype=torch.long, pin_memory=pin)
+            self.h_pos32 = torch.zeros(mb, dtype=torch.int32, pin_memory=pin)
+            self.n_prev = self.h_prev.numpy()
+            self.n_pos32 = self.h_pos32.numpy()
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.outs: dict[int, torch.Tensor] = {}
         self.metas: dict[int, ForwardMeta] = {}
 
     def _meta(self, bs: int) -> ForwardMeta:
-        return ForwardMeta(
+        meta = ForwardMeta(
             is_prefill=False,
             positions=self.positions[:bs],
             slot_mapping=self.slots[:bs],
@@ -86,6 +98,15 @@ class DecodeGraphRunner:
             block_tables=self.block_tables[:bs],
             seq_lens=self.seq_lens[:bs],
         )
+        if self.ragged:
+            meta.ragged = RaggedMeta(
+                block_tables=self.block_tables[:bs],
+                row_seq=self.row_seq[:bs], pos32=self.pos32[:bs],
+                prev_tokens=self.prev[:bs], seq_starts=list(range(bs)),
+                seq_hists=[0] * bs, seq_news=[1] * bs,
+                # static launch shape: split for the longest context
+                max_ctx=self.runner.cfg.max_model_len)
+        return meta
 
     def capture(self) -> None:
         model, kv = self.runner.model, self.runner.kv
@@ -122,6 +143,14 @@ class DecodeGraphRunner:
         self.n_positions[:bs] = batch.positions
         self.n_slots[:bs] = batch.slot_mapping
         self.n_seq_lens[:bs] = np.asarray(batch.seq_lens, dtype=np.int32)
+        if self.ragged:
+            self.n_pos32[:bs] = np.asarray(batch.positions, dtype=np.int32)
+            for si, s in enumerate(batch.seqs):
+                r0 = si * rps
+                p0 = int(batch.positions[r0])
+                self.n_prev[r0] = s.all_token_ids[p0 - 1] if p0 > 0 else -1
+                for j in range(1, rps):
+                    self.n_prev[r0 + j] = batch.token_ids[r0 + j - 1]
         maxb = 0
         dirty_lo, dirty_hi = self.max_bs, -1
         for si, s in enumerate(batch.seqs):
@@ -143,6 +172,9 @@ class DecodeGraphRunner:
             self.n_slots[bs:hi] = self._pad_slot
             self.n_seq_lens[bs:hi] = 1
             self.h_bt[bs:hi, 0] = self.pad_block
+            if self.ragged:
+                self.n_pos32[bs:hi] = 0
+                self.n_prev[bs:hi] = -1
             for i in range(bs, hi):
                 self._row_state[i] = None
             dirty_lo = min(dirty_lo, bs)
@@ -160,6 +192,9 @@ class DecodeGraphRunner:
         self.positions[:n].copy_(self.h_positions[:n], non_blocking=True)
         self.slots[:n].copy_(self.h_slots[:n], non_blocking=True)
         self.seq_lens[:n].copy_(self.h_seq_lens[:n], non_blocking=True)
+        if self.ragged:
+            self.pos32[:n].copy_(self.h_pos32[:n], non_blocking=True)
+            self.prev[:n].copy_(self.h_prev[:n], non_blocking=True)
         if dirty_hi >= 0:
             self.block_tables[dirty_lo:dirty_hi + 1, :max(maxb, 1)].copy_(
                 self.h_bt[dirty_lo:dirty_hi + 1, :max(maxb, 1)], non_blocking=True

@@ -148,7 +148,22 @@ class KVCache:
         # (v_caches stay as zero-size placeholders so the layer-forward
         # signature is uniform)
         self.mla = bool(spec.kv_lora_rank)
-        if self.mla:
+        # heterogeneous latent stacks (spec.layers): layer i's pool is
+        # [nblocks, P, BS, kv_rank_i] in the engine dtype — widths may
+        # differ per layer while block ids stay shared, so one block table
+        # still drives every layer. bf16 pools hold every page twice
+        # (P = 2: row-major and transposed) so both MFMA products of
+        # ops.latent_attention reduce over a contiguous axis; that is still
+        # 2 * kv_rank values per token against heads * (qk + v) expanded
+        self.layered = spec.layers is not None
+        if self.layered:
+            kv_heads = 1
+            self.kv_heads = 1
+            self.mla = True     # latent-only pool: no V pool, no host tier
+            if cfg.kv_cache_dtype == "fp8":
+                raise ValueError("fp8 KV is not supported with latent pools")
+            shape = None
+        elif self.mla:
             kv_heads = 1
             self.kv_heads = 1
             lat = spec.kv_lora_rank + spec.qk_rope_head_dim
@@ -160,9 +175,18 @@ class KVCache:
         else:
             dtype = getattr(torch, cfg.dtype)
         self.kv_dtype = dtype
-        self.k_caches = [
-            torch.zeros(shape, dtype=dtype, device=device) for _ in range(self.num_layers)
-        ]
+        if self.layered:
+            self.k_caches = [
+                torch.zeros((num_blocks, self.latent_planes(cfg),
+                             cfg.block_size, ls.mixer.kv_rank),
+                            dtype=dtype, device=device)
+                for ls in spec.layers[:self.num_layers]
+            ]
+        else:
+            self.k_caches = [
+                torch.zeros(shape, dtype=dtype, device=device)
+                for _ in range(self.num_layers)
+            ]
         if self.mla:
             self.v_caches = [
                 torch.zeros(0, dtype=dtype, device=device)
@@ -203,6 +227,10 @@ class KVCache:
             self.host_pool = None
             self.host_allocator = None
             self.side_stream = None
+
+    @staticmethod
+    def latent_planes(cfg: EngineConfig) -> int:
+        return 2 if cfg.dtype == "bfloat16" else 1
 
     # ---- offload tier ----------------------------------------------------
 
@@ -264,7 +292,11 @@ class KVCache:
         nl = num_layers if num_layers is not None else spec.num_layers
         kv_heads = max(1, spec.num_kv_heads // cfg.tp_size)
         esize = 1 if cfg.kv_cache_dtype == "fp8" else 2
-        if spec.kv_lora_rank:
+        if spec.layers is not None:
+            esize = 4 if cfg.dtype == "float32" else 2
+            per_block = (cfg.block_size * spec.kv_bytes_per_token(esize)
+                         * KVCache.latent_planes(cfg))
+        elif spec.kv_lora_rank:
             per_block = (nl * cfg.block_size
                          * (spec.kv_lora_rank + spec.qk_rope_head_dim)
                          * esize)

@@ -218,7 +218,8 @@ class ModelRunner:
         self.comm = comm or Communicator()
         self.cp_prefills = 0
         self.cp_suffixes = 0
-        if torch.device(cfg.device).type == "cuda" and (
+        if torch.device(cfg.device).type == "cuda" \
+                and cfg.spec.layers is None and (
                 cfg.spec.attention_sinks or cfg.spec.sliding_window
                 or cfg.spec.attn_logit_softcap
                 or cfg.spec.norm_type != "rmsnorm"
@@ -255,7 +256,11 @@ class ModelRunner:
         if self.device.type == "cuda":
             self._init_tunableop()
         self.graph_runner = None
-        self.model = LlamaForCausalLM(cfg, self.comm, self.device)
+        from ..models import model_class_for
+
+        self.model = model_class_for(cfg.spec.architecture)(
+            cfg, self.comm, self.device)
+        self.ragged = bool(getattr(self.model, "uses_ragged_meta", False))
         if cfg.gguf_path and not cfg.enforce_random_weights:
             from ..models.weights import load_gguf
 
@@ -399,7 +404,9 @@ class ModelRunner:
             eagle_graphs = (self.eagle is not None
                             and os.environ.get("GPUSTACK_AMD_EAGLE_GRAPHS",
                                                "0") == "1")
-            if graphs_enabled() and moe_graph_ok \
+            ragged_ok = (not self.ragged
+                         or self.model.graph_capturable())
+            if graphs_enabled() and moe_graph_ok and ragged_ok \
                     and (self.eagle is None or eagle_graphs) \
                     and self.comm.pp_size == 1 \
                     and self.model.offload is None:
@@ -542,7 +549,69 @@ class ModelRunner:
         )
         return tokens, meta
 
+    def _ragged_meta(self, batch: ScheduledBatch, positions) -> "RaggedMeta":
+        """The per-sequence (first row, cached tokens, rows) view of any
+        batch kind plus each row's previous token (RaggedMeta)."""
+        from ..models.llama import RaggedMeta
+
+        dev = self.device
+        pos = [int(p) for p in batch.positions]
+        toks = [int(t) for t in batch.token_ids]
+        if batch.is_prefill:
+            n_pre = batch.n_prefill_seqs or len(batch.seqs)
+            news = list(batch.seq_lens[:n_pre]) + [1] * (len(batch.seqs) - n_pre)
+        elif batch.is_suffix:
+            news = list(batch.suffix_rows)
+        else:
+            news = [batch.rows_per_seq] * len(batch.seqs)
+        starts, hists, row_seq, prev = [], [], [], []
+        off = 0
+        for i, (s, n) in enumerate(zip(batch.seqs, news)):
+            starts.append(off)
+            hists.append(pos[off])
+            row_seq.extend([i] * n)
+            p0 = pos[off]
+            # the token before the portion's first row is part of the
+            # sequence's own record; inside the portion it is the row before
+            prev.append(s.all_token_ids[p0 - 1] if p0 > 0 else -1)
+            prev.extend(toks[off:off + n - 1])
+            off += n
+        maxb = max(len(s.block_table) for s in batch.seqs)
+        bt = torch.zeros(len(batch.seqs), maxb, dtype=torch.int32)
+        for i, s in enumerate(batch.seqs):
+            bt[i, : len(s.block_table)] = torch.tensor(s.block_table,
+                                                       dtype=torch.int32)
+        return RaggedMeta(
+            block_tables=bt.to(dev),
+            row_seq=torch.tensor(row_seq, dtype=torch.int32, device=dev),
+            pos32=positions.to(torch.int32),
+            prev_tokens=torch.tensor(prev, dtype=torch.long, device=dev),
+            seq_starts=starts, seq_hists=hists, seq_news=news,
+            max_ctx=max(h + n for h, n in zip(hists, news)))
+
     def _meta(self, batch: ScheduledBatch) -> tuple[torch.Tensor, ForwardMeta]:
+        tokens, meta = self._meta_by_kind(batch)
+        if batch.logit_rows is not None:
+            meta.logits_indices = torch.tensor(
+                batch.logit_rows, dtype=torch.long, device=self.device)
+        if self.ragged:
+            meta.ragged = self._ragged_meta(batch, meta.positions)
+        return tokens, meta
+
+    @torch.inference_mode()
+    def forward_logits(self, batch: ScheduledBatch) -> torch.Tensor:
+        """Run one scheduled batch and return the fp32 logits of its
+        logit rows without sampling (forced-token replay, scoring)."""
+        tokens, meta = self._meta(batch)
+        if meta.logits_indices.numel() == 0:
+            # nothing asked for: the step still has to fill the cache
+            meta.logits_indices = torch.zeros(1, dtype=torch.long,
+                                              device=self.device)
+            self.model(tokens, meta, self.kv)
+            return torch.empty(0, self.cfg.spec.vocab_size)
+        return self.model(tokens, meta, self.kv).float()
+
+    def _meta_by_kind(self, batch: ScheduledBatch) -> tuple[torch.Tensor, ForwardMeta]:
         if self._cp_splittable(batch):
             return self._meta_cp(batch)
         dev = self.device

@@ -47,6 +47,9 @@ class ScheduledBatch:
     # an intermediate chunk whose sampled token must be discarded and whose
     # seq must not yet join the running set
     chunk_final: list[bool] | None = None
+    # explicit rows whose logits the step returns (forced-token replay and
+    # scoring); None = the batch kind's default (last row of every seq)
+    logit_rows: list[int] | None = None
 
     @property
     def num_tokens(self) -> int:
@@ -421,6 +424,47 @@ class Scheduler:
         if final:
             self._chunking = None
         return batch
+
+    def schedule_forced(self, plan: "list[tuple[Sequence, int, list[int]]]"
+                        ) -> ScheduledBatch:
+        """Forced-token step: run exactly the next `n` recorded tokens of
+        every listed sequence together as ONE batch — prompt portions of
+        any size beside single tokens — from the KV each sequence already
+        holds. plan entries are (seq, n, wanted) with `wanted` the local
+        rows whose logits are returned. Nothing is sampled and no sequence
+        joins the running set; blocks come from (and, through release(),
+        return to) the same pool the generation path uses."""
+        batch = ScheduledBatch(is_prefill=False, is_suffix=True)
+        batch.suffix_rows, batch.chunk_final, batch.logit_rows = [], [], []
+        toks, poss, slots, lens = [], [], [], []
+        for seq, n, wanted in plan:
+            p = seq.num_cached_tokens
+            tokens = seq.all_token_ids
+            if n <= 0 or p + n > len(tokens):
+                raise ValueError("forced step outside the sequence's tokens")
+            need = self.kv.blocks_needed(p + n) - len(seq.block_table)
+            if need > 0:
+                seq.block_table.extend(self.kv.allocator.allocate(need))
+            seq.status = SeqStatus.RUNNING
+            base = len(toks)
+            batch.seqs.append(seq)
+            batch.suffix_rows.append(n)
+            batch.chunk_final.append(False)
+            batch.logit_rows.extend(base + int(w) for w in wanted)
+            toks.extend(tokens[p:p + n])
+            poss.extend(range(p, p + n))
+            slots.extend(self.kv.slots_for(seq.block_table, p, n))
+            lens.extend(range(p + 1, p + n + 1))
+            seq.num_cached_tokens = p + n
+        batch.token_ids, batch.positions = toks, poss
+        batch.slot_mapping, batch.seq_lens = slots, lens
+        batch.n_prefill_seqs = len(batch.seqs)
+        return batch
+
+    def release(self, seq: Sequence) -> None:
+        """Give back everything a forced-step sequence holds."""
+        self._release(seq)
+        seq.num_cached_tokens = 0
 
     def _schedule_decode(self) -> ScheduledBatch | None:
         if not self.running:
