@@ -3,6 +3,7 @@
   python -m gpustack_amd start [--config FILE] [flags]           # server
   python -m gpustack_amd start --server-url http://... --token T # worker
   python -m gpustack_amd chat --model NAME --prompt "..."        # client
+  python -m gpustack_amd replay --model DIR --out DIR --max-tokens N  # trace
   python -m gpustack_amd version
 """
 from __future__ import annotations
@@ -52,8 +53,25 @@ def main(argv: list[str] | None = None) -> int:
     kp.add_argument("--bootstrap-password", default="admin")
     kp.add_argument("--registration-token", default="tok_cluster")
     kp.add_argument("--gpus-per-node", type=int, default=8)
+    tp = sub.add_parser(
+        "replay", help="replay recorded token steps (JSON lines on stdin) "
+        "through the engine and write the wanted logits")
+    tp.add_argument("--model", required=True,
+                    help="folder with config.json and model.safetensors")
+    tp.add_argument("--dtype", default="bfloat16",
+                    choices=["bfloat16", "float32"])
+    tp.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    tp.add_argument("--max-tokens", dest="max_tokens", type=int, required=True,
+                    help="tokens the live requests hold at most (pool size)")
+    tp.add_argument("--device", default=None)
     sub.add_parser("version")
     args = ap.parse_args(argv)
+
+    if args.cmd == "replay":
+        from .engine.replay import run_trace
+
+        return run_trace(args.model, args.dtype, args.out, args.max_tokens,
+                         device=args.device)
 
     if args.cmd == "manifests":
         from .utils.k8s_manifests import render_all
