@@ -55,11 +55,25 @@ def parse_args():
     ap.add_argument("--cp", type=int, default=1,
                     help="prefill-context-parallel degree (rows chunked "
                          "across ranks, replicated decode); world = tp*cp")
+    ap.add_argument("--layer-bench", action="store_true",
+                    help="instead of the serving workload: Vunitar layers at "
+                         "real-model sizes beside the closest llama-lineage "
+                         "stack (prefill/decode tok/s + per-kernel roofline "
+                         "shares; gpustack_amd/bench/layer_bench.py)")
+    ap.add_argument("--layer-sizes", default="small,medium",
+                    help="comma list of small,medium,large for --layer-bench")
     return ap.parse_args()
 
 
 def main():
     args = parse_args()
+    if args.layer_bench:
+        from gpustack_amd.bench.layer_bench import run as run_layer_bench
+
+        run_layer_bench(args.layer_sizes.split(","),
+                        args.device or ("cuda:0" if torch.cuda.is_available()
+                                        else "cpu"))
+        return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     local_rank = int(os.environ.get("LOCAL_RANK", str(rank)))
