@@ -443,3 +443,46 @@ def test_greedy_generation(small):
     eng2.cfg.max_prefill_tokens = 8
     assert eng2.generate([prompts[1]], SamplingParams(
         max_tokens=6, ignore_eos=True))[0] == outs[1][:6]
+
+
+# ---- the replay command line ---------------------------------------------------
+
+def test_trace_replay_command(small, tmp_path):
+    """bin/trace_run: JSON steps on stdin, `done <step>` lines on stdout,
+    <step>.f32 files with the wanted logits; a pool of max-tokens is enough
+    because ended requests give their blocks back."""
+    import subprocess
+
+    import numpy as np
+
+    cfg, w, d = small
+    a, b = toks(40, cfg["vocab"], 50), toks(35, cfg["vocab"], 51)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}],
+         "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[30:39], "want": []}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[39:], "want": [0]}],
+         "end": ["a"]},
+        {"step": 3, "entries": [{"id": "b", "tokens": b, "want": [34, 3]}],
+         "end": ["b"]},
+    ]
+    out = tmp_path / "out"
+    exe = Path(__file__).resolve().parent.parent / "bin" / "trace_run"
+    r = subprocess.run(
+        [sys.executable, str(exe), "--model", d, "--dtype", "float32",
+         "--out", str(out), "--max-tokens", "64", "--device", "cpu"],
+        input="".join(json.dumps(s) + "\n" for s in steps),
+        capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    done = [ln for ln in r.stdout.splitlines() if ln.startswith("done ")]
+    assert done == ["done 0", "done 1", "done 2", "done 3"]
+    assert not (out / "1.f32").exists()
+    wa, wb = oracle.forward(cfg, w, a), oracle.forward(cfg, w, b)
+    V = cfg["vocab"]
+    got0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(-1, V))
+    close(got0, wa[[0, 29]])
+    got2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(-1, V))
+    close(got2, wa[[39]])
+    got3 = torch.from_numpy(np.fromfile(out / "3.f32", dtype="<f4").reshape(-1, V))
+    close(got3, wb[[34, 3]])
