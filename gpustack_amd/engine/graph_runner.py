@@ -148,7 +148,7 @@ class DecodeGraphRunner:
             for si, s in enumerate(batch.seqs):
                 r0 = si * rps
                 p0 = int(batch.positions[r0])
-                self.n_prev[r0] = s.all_token_ids[p0 - 1] if p0 > 0 else -1
+                self.n_prev[r0] = s.token_at(p0 - 1) if p0 > 0 else -1
                 for j in range(1, rps):
                     self.n_prev[r0 + j] = batch.token_ids[r0 + j - 1]
         maxb = 0

@@ -554,9 +554,11 @@ class ModelRunner:
         batch kind plus each row's previous token (RaggedMeta)."""
         from ..models.llama import RaggedMeta
 
+        import numpy as np
+
         dev = self.device
-        pos = [int(p) for p in batch.positions]
-        toks = [int(t) for t in batch.token_ids]
+        pos = np.asarray(batch.positions, dtype=np.int64)
+        toks = np.asarray(batch.token_ids, dtype=np.int64)
         if batch.is_prefill:
             n_pre = batch.n_prefill_seqs or len(batch.seqs)
             news = list(batch.seq_lens[:n_pre]) + [1] * (len(batch.seqs) - n_pre)
@@ -564,18 +566,16 @@ class ModelRunner:
             news = list(batch.suffix_rows)
         else:
             news = [batch.rows_per_seq] * len(batch.seqs)
-        starts, hists, row_seq, prev = [], [], [], []
-        off = 0
-        for i, (s, n) in enumerate(zip(batch.seqs, news)):
-            starts.append(off)
-            hists.append(pos[off])
-            row_seq.extend([i] * n)
-            p0 = pos[off]
-            # the token before the portion's first row is part of the
-            # sequence's own record; inside the portion it is the row before
-            prev.append(s.all_token_ids[p0 - 1] if p0 > 0 else -1)
-            prev.extend(toks[off:off + n - 1])
-            off += n
+        starts = np.concatenate(([0], np.cumsum(news)[:-1])).astype(np.int64)
+        hists = pos[starts]
+        # inside a portion the previous token is the row before; the token
+        # before a portion's first row comes from the sequence's own record
+        prev = np.empty(len(toks), dtype=np.int64)
+        prev[1:] = toks[:-1]
+        for s, st, p0 in zip(batch.seqs, starts.tolist(), hists.tolist()):
+            prev[st] = s.token_at(p0 - 1) if p0 > 0 else -1
+        row_seq = np.repeat(np.arange(len(news), dtype=np.int32), news)
+        starts, hists = starts.tolist(), hists.tolist()
         maxb = max(len(s.block_table) for s in batch.seqs)
         bt = torch.zeros(len(batch.seqs), maxb, dtype=torch.int32)
         for i, s in enumerate(batch.seqs):
@@ -583,9 +583,9 @@ class ModelRunner:
                                                        dtype=torch.int32)
         return RaggedMeta(
             block_tables=bt.to(dev),
-            row_seq=torch.tensor(row_seq, dtype=torch.int32, device=dev),
+            row_seq=torch.from_numpy(row_seq).to(dev),
             pos32=positions.to(torch.int32),
-            prev_tokens=torch.tensor(prev, dtype=torch.long, device=dev),
+            prev_tokens=torch.from_numpy(prev).to(dev),
             seq_starts=starts, seq_hists=hists, seq_news=news,
             max_ctx=max(h + n for h, n in zip(hists, news)))
 

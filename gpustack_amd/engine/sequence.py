@@ -99,6 +99,12 @@ class Sequence:
     def all_token_ids(self) -> list[int]:
         return self.prompt_token_ids + self.output_token_ids
 
+    def token_at(self, i: int) -> int:
+        """Token id at absolute position i without building the full list."""
+        n = len(self.prompt_token_ids)
+        return (self.prompt_token_ids[i] if i < n
+                else self.output_token_ids[i - n])
+
     @property
     def num_prompt_tokens(self) -> int:
         return len(self.prompt_token_ids)

@@ -432,20 +432,31 @@ def build_latent_tiles(seq_starts, seq_hists, seq_news, heads: int, device):
     latents once for all of them. Long portions tile as 16 rows x 1 head;
     short ones (decode rows above all) pack rows x heads. Returns int32
     [ntiles, 6]: row0, nrows, head0, nheads, seq, pos0."""
-    tiles = []
+    import numpy as np
+
     G = _LAT_GROUP
+    parts = []
     for i, (st, hist, new) in enumerate(zip(seq_starts, seq_hists, seq_news)):
         if new >= G:
             nh, nr = 1, G
         else:
             nh = min(heads, G)
             nr = max(1, min(new, G // nh))
-        for r0 in range(0, new, nr):
-            n = min(nr, new - r0)
-            for h0 in range(0, heads, nh):
-                tiles.append((st + r0, n, h0, min(nh, heads - h0), i,
-                              hist + r0))
-    return torch.tensor(tiles, dtype=torch.int32, device=device).view(-1, 6)
+        r0 = np.arange(0, new, nr, dtype=np.int32)
+        h0 = np.arange(0, heads, nh, dtype=np.int32)
+        rr, hh = np.meshgrid(r0, h0, indexing="ij")
+        rr, hh = rr.reshape(-1), hh.reshape(-1)
+        t = np.empty((rr.size, 6), dtype=np.int32)
+        t[:, 0] = st + rr
+        t[:, 1] = np.minimum(nr, new - rr)
+        t[:, 2] = hh
+        t[:, 3] = np.minimum(nh, heads - hh)
+        t[:, 4] = i
+        t[:, 5] = hist + rr
+        parts.append(t)
+    tiles = (np.concatenate(parts) if parts
+             else np.empty((0, 6), dtype=np.int32))
+    return torch.from_numpy(tiles).to(device)
 
 
 def latent_attention_mfma_ok(cache) -> bool:
