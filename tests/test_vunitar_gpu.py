@@ -31,6 +31,27 @@ STEPS = [[("a", 17), ("b", 2)], [("a", 1), ("b", 1), ("c", 16), ("d", 1)],
          [("a", 30), ("c", 1)], [("c", 4), ("a", 1)], [("a", 1)]]
 
 
+@pytest.fixture
+def gpu_engine():
+    """Engine factory whose engines are torn down when the test is over:
+    an engine is a reference cycle (runner <-> graph runner), so without an
+    explicit collection its captured graphs and pool would linger into
+    whatever runs next in the process."""
+    import gc
+
+    made = []
+
+    def make(model_dir, **kw):
+        made.append(tv.make_engine(model_dir, device="cuda", **kw))
+        return made[-1]
+
+    yield make
+    made.clear()
+    gc.collect()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+
+
 def _model(tmp_path, kw, seed=3):
     cfg = tv.make_config(**kw)
     w = tv.make_weights(cfg, seed=seed)
@@ -38,19 +59,19 @@ def _model(tmp_path, kw, seed=3):
 
 
 @pytest.mark.parametrize("name", ["default", "wide", "aligned"])
-def test_fp32_engine_matches_oracle(tmp_path, name):
+def test_fp32_engine_matches_oracle(tmp_path, gpu_engine, name):
     kw = {"default": {}, "wide": tv.VARIANTS["wide"], "aligned": ALIGNED}[name]
     cfg, w, d = _model(tmp_path, kw)
-    eng = tv.make_engine(d, device="cuda")
+    eng = gpu_engine(d)
     reqs = {i: tv.toks(n, cfg["vocab"], 70 + n) for i, n in REQS.items()}
     got = tv.run_schedule(eng, reqs, STEPS)
     for i, t in reqs.items():
         tv.close(got[i], oracle.forward(cfg, w, t), 2e-3)
 
 
-def test_bf16_engine_mfma_and_grouped_experts(tmp_path):
+def test_bf16_engine_mfma_and_grouped_experts(tmp_path, gpu_engine):
     cfg, w, d = _model(tmp_path, ALIGNED)
-    eng = tv.make_engine(d, dtype="bfloat16", device="cuda", blocks=12)
+    eng = gpu_engine(d, dtype="bfloat16", blocks=12)
     assert ops._load_latent().latent_attention_uses_mfma(eng.runner.kv.k_caches[0])
     for rnd in range(3):      # blocks are freed and taken again
         reqs = {i: tv.toks(n, cfg["vocab"], 80 + n + rnd) for i, n in REQS.items()}
@@ -64,7 +85,7 @@ def test_bf16_engine_mfma_and_grouped_experts(tmp_path):
 
 @pytest.mark.parametrize("dtype,R", [("float32", 8), ("bfloat16", 8),
                                      ("bfloat16", 32)])
-def test_far_keys_and_page_borders(tmp_path, dtype, R):
+def test_far_keys_and_page_borders(tmp_path, gpu_engine, dtype, R):
     T = 200
     targets = {150: [0, 1], 151: [15, 16], 152: [17, 31], 153: [32, 47],
                160: [48, 63], 175: [64, 127], 176: [128, 143], 177: [144, 149],
@@ -73,7 +94,7 @@ def test_far_keys_and_page_borders(tmp_path, dtype, R):
     t = list(range(T))
     want = oracle.forward(cfg, w, t)
     rows = sorted(targets)
-    eng = tv.make_engine(d, dtype=dtype, device="cuda")
+    eng = gpu_engine(d, dtype=dtype)
     tol = 2e-3 if dtype == "float32" else 0.15
     tv.close(tv.run_schedule(eng, {"a": t}, [[("a", T)]])["a"][rows], want[rows], tol)
     cut = [16, 15, 2, 31, 64, 23, 2, 16, 7, 24]
@@ -84,12 +105,12 @@ def test_far_keys_and_page_borders(tmp_path, dtype, R):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_generation_agrees_with_replay(tmp_path, dtype):
+def test_generation_agrees_with_replay(tmp_path, gpu_engine, dtype):
     """Greedy generation (scheduler, decode batches; captured graphs for the
     bf16 engine) must pick the tokens that the forced-token path scores
     highest at the same places."""
     cfg, w, d = _model(tmp_path, ALIGNED)
-    eng = tv.make_engine(d, dtype=dtype, device="cuda", blocks=64, max_seqs=8)
+    eng = gpu_engine(d, dtype=dtype, blocks=64, max_seqs=8)
     if dtype == "bfloat16":
         assert eng.runner.graph_runner is not None
     prompts = [tv.toks(n, cfg["vocab"], 90 + n) for n in (9, 20, 1, 33)]
