@@ -127,7 +127,9 @@ def reshape_and_cache(k, v, k_cache, v_cache, slots) -> None:
 
 def greedy_sample_into(out, logits) -> None:
     if logits.is_cuda and logits.dtype == torch.float32:
-        _load_latent().argmax_f32(out, logits)  # fp32-logit models
+        # fp32-logit models: whichever fp32-stream library is loaded
+        (_PAGED if _PAGED is not None else _load_latent()).argmax_f32(
+            out, logits)
         return
     hip = _backend(logits)
     if hip is not None:
@@ -359,6 +361,32 @@ build_cos_sin_cache = torch_ref.build_cos_sin_cache
 # instantiated for both.
 
 _LATENT = None
+_PAGED = None
+
+
+def _load_paged():
+    """Load `_hip_paged.so` (row kernels of the pre/post-norm fp32 stream
+    and paged rotary attention), compiling it in-tree first when no built
+    library is there."""
+    global _PAGED
+    if _PAGED is not None:
+        return _PAGED
+    import importlib.util
+
+    from .build import PAGED_SO_PATH, build_paged
+
+    if not PAGED_SO_PATH.exists():
+        build_paged()
+    spec = importlib.util.spec_from_file_location(
+        "gpustack_amd.ops._hip_paged", PAGED_SO_PATH)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    _PAGED = mod
+    return mod
+
+
+def _paged_backend(t: torch.Tensor):
+    return _load_paged() if t.is_cuda else None
 
 
 def _load_latent():
@@ -541,3 +569,160 @@ def softcap_(logits, cap: float) -> None:
         k.softcap(logits, cap)
     else:
         torch_ref.softcap_(logits, cap)
+
+
+# --- pre/post-norm fp32 stream + paged rotary attention -------------------
+# ops/csrc/rowmix32.hip and ops/csrc/ragged_attn.hip in `_hip_paged.so`.
+
+def embed_rows_f32(x, tokens, embed) -> None:
+    k = _paged_backend(x)
+    if k is not None:
+        k.embed_rows_f32(x, tokens, embed)
+    else:
+        torch_ref.embed_rows_f32(x, tokens, embed)
+
+
+def rms_norm_rows(out, x, weight, eps: float) -> None:
+    """fp32 rows -> weighted RMS norm in out's dtype."""
+    k = _paged_backend(x)
+    if k is not None:
+        k.sandwich_add_norm(x, None, None, 0.0, eps, None, weight, out)
+    else:
+        torch_ref.rms_norm_f32(out, x, weight, eps)
+
+
+def sandwich_add_norm(x, a, post_w, mult: float, eps: float, extra, next_w,
+                      h) -> None:
+    k = _paged_backend(x)
+    if k is not None:
+        k.sandwich_add_norm(x, a, post_w, mult, eps, extra, next_w, h)
+    else:
+        torch_ref.sandwich_add_norm(x, a, post_w, mult, eps, extra, next_w, h)
+
+
+def build_page_groups(seq_starts, seq_hists, seq_news, block_size: int,
+                      device):
+    """Runs of batch rows that fall into ONE cache page in order, for
+    page-wise value stores: int32 [n, 2] = first row, rows. A sequence that
+    brings rows for positions hist..hist+new-1 is cut at multiples of the
+    page size."""
+    import numpy as np
+
+    parts = []
+    for st, hist, new in zip(seq_starts, seq_hists, seq_news):
+        first = np.arange(hist - hist % block_size, hist + new, block_size)
+        lo = np.maximum(first, hist)
+        hi = np.minimum(first + block_size, hist + new)
+        parts.append(np.stack([st + lo - hist, hi - lo], axis=1))
+    g = (np.concatenate(parts) if parts else np.empty((0, 2))).astype(np.int32)
+    return torch.from_numpy(g).to(device)
+
+
+def rotary_norm_store(q_out, qkv, nq: int, nk: int, q_norm_w, k_norm_w,
+                      inv_freq, pos32, head_dim: int, k_cache, v_cache, slots,
+                      eps: float, tied: bool, page_groups=None) -> None:
+    """`page_groups` (build_page_groups; GPU, prompts): the value rows are
+    written page by page instead of row by row."""
+    k = _paged_backend(qkv)
+    if k is not None:
+        k.rotary_norm_store(q_out, qkv, nq, nk, q_norm_w, k_norm_w, inv_freq,
+                            pos32, head_dim, k_cache, v_cache, slots, eps,
+                            tied, page_groups)
+    else:
+        torch_ref.rotary_norm_store(q_out, qkv, nq, nk, q_norm_w, k_norm_w,
+                                    inv_freq, pos32, head_dim, k_cache,
+                                    v_cache, slots, eps, tied)
+
+
+_ATT_GROUP = 16   # (row, score map) pairs sharing one key stream per workgroup
+
+
+def build_attn_tiles(seq_starts, seq_hists, seq_news, heads: int,
+                     kv_heads: int, maps: int, device):
+    """Group the batch's (row, score map) pairs into tiles of at most 16
+    pairs that share ONE key stream: same sequence, same kv head, same map.
+    Long portions tile as 16 rows x 1 query head; short ones (decode rows
+    above all) pack rows x the query heads of a kv group. Score map a =
+    head * maps + map, so the heads of one kv group and one map are `maps`
+    apart. Returns int32 [ntiles, 6]: row0, nrows, a0, n_a, seq, a_step."""
+    import numpy as np
+
+    G = _ATT_GROUP
+    rep = heads // kv_heads
+    parts = []
+    for i, (st, hist, new) in enumerate(zip(seq_starts, seq_hists, seq_news)):
+        if new >= G or rep == 1:
+            nh, nr = 1, G
+        else:
+            nh = min(rep, G)
+            nr = max(1, min(new, G // nh))
+        r0 = np.arange(0, new, nr, dtype=np.int32)
+        # first score map of every (kv head, chunk of nh heads, map)
+        g0 = np.arange(0, rep, nh, dtype=np.int32)
+        a0 = ((np.arange(kv_heads, dtype=np.int32)[:, None, None] * rep
+               + g0[None, :, None]) * maps
+              + np.arange(maps, dtype=np.int32)[None, None, :])
+        na = np.broadcast_to(np.minimum(nh, rep - g0)[None, :, None],
+                             a0.shape).reshape(-1)
+        a0 = a0.reshape(-1)
+        rr, ai = np.meshgrid(r0, np.arange(a0.size), indexing="ij")
+        rr, ai = rr.reshape(-1), ai.reshape(-1)
+        t = np.empty((rr.size, 6), dtype=np.int32)
+        t[:, 0] = st + rr
+        t[:, 1] = np.minimum(nr, new - rr)
+        t[:, 2] = a0[ai]
+        t[:, 3] = na[ai]
+        t[:, 4] = i
+        t[:, 5] = maps
+        parts.append(t)
+    tiles = (np.concatenate(parts) if parts
+             else np.empty((0, 6), dtype=np.int32))
+    return torch.from_numpy(tiles).to(device)
+
+
+def paged_attention(out, q, k_cache, v_cache, block_tables, row_seq, positions,
+                    scale: float, maps: int = 1, window: int = 0,
+                    keep_first: int = 0, sinks=None, tiles=None,
+                    exact: bool = False, max_ctx: int = 0) -> None:
+    """q: [T, A, D], out: [T, A, VW] (A = heads * maps score maps). On the
+    GPU the MFMA kernel runs for bf16 pools of fitting sizes, the fp32
+    vector-ALU kernel otherwise (always for fp32 pools, or with `exact`).
+    `max_ctx` (longest context in the batch, a host number) lets a batch of
+    few tiles over long contexts split each tile's keys over workgroups."""
+    k = _paged_backend(q)
+    if k is not None:
+        if tiles is None:
+            raise ValueError("paged_attention on GPU needs the tile list "
+                             "(build_attn_tiles)")
+        nsplit = 1
+        nt = tiles.shape[0]
+        span = min(max_ctx, window + keep_first) if window > 0 else max_ctx
+        if span >= 512 and 0 < nt < 2048:
+            # 1024 workgroups, or up to 2048 while the split stays <= 4 (a
+            # wider split pays more for the merge than it gains in
+            # occupancy), each of at least 128 keys
+            nsplit = max(1, min(16, span // 128,
+                                max(1024 // nt, min(4, 2048 // nt))))
+        k.paged_attention(out, q, k_cache, v_cache, block_tables, tiles,
+                          positions, scale, maps, window, keep_first, sinks,
+                          exact, nsplit)
+    else:
+        torch_ref.paged_attention(out, q, k_cache, v_cache, block_tables,
+                                  row_seq, positions, scale, maps, window,
+                                  keep_first, sinks)
+
+
+def diff_combine(out, a, lam, diff: float, eps: float) -> None:
+    k = _paged_backend(a)
+    if k is not None:
+        k.diff_combine(out, a, lam, diff, eps)
+    else:
+        torch_ref.diff_combine(out, a, lam, diff, eps)
+
+
+def act_and_mul(out, gu, mode: str) -> None:
+    k = _paged_backend(gu)
+    if k is not None:
+        k.act_and_mul(out, gu, ACT_MODES[mode])
+    else:
+        torch_ref.act_and_mul(out, gu, mode)

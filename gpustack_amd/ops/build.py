@@ -27,6 +27,13 @@ LATENT_SOURCES = ["resid32.hip", "latent_attn.hip", "grouped_ff.hip",
                   "latent_bindings.cpp"]
 
 
+# pre/post-norm fp32-stream row kernels + paged rotary attention (argmax
+# comes with resid32.hip): again a library of its own
+PAGED_SO_PATH = PKG_DIR / "_hip_paged.so"
+PAGED_SOURCES = ["rowmix32.hip", "ragged_attn.hip", "resid32.hip",
+                 "paged_bindings.cpp"]
+
+
 def _torch_paths():
     import torch
 
@@ -130,21 +137,34 @@ def build(verbose: bool = False, force: bool = False) -> Path:
 
 
 def build_latent(verbose: bool = False, force: bool = True) -> Path:
-    """Compile the fp32-residual op family into `_hip_latent.so`. Objects
-    are built under a private name and the library is moved into place at
-    the end, so a concurrent reader never sees a half-written file."""
+    """Compile the fp32-residual op family into `_hip_latent.so`."""
+    return _build_small("_hip_latent", LATENT_SOURCES, LATENT_SO_PATH,
+                        verbose, force)
+
+
+def build_paged(verbose: bool = False, force: bool = True) -> Path:
+    """Compile the paged rotary attention family into `_hip_paged.so`."""
+    return _build_small("_hip_paged", PAGED_SOURCES, PAGED_SO_PATH,
+                        verbose, force)
+
+
+def _build_small(ext_name: str, sources: list[str], so_path: Path,
+                 verbose: bool, force: bool) -> Path:
+    """Compile one small extension, its files in parallel. Objects are
+    built under a private name and the library is moved into place at the
+    end, so a concurrent reader never sees a half-written file."""
     includes, libdir, abi = _torch_paths()
     inc_flags = [f"-I{p}" for p in includes]
-    flags = _common_flags(abi, "_hip_latent")
-    build_dir = CSRC / ".build_latent"
+    flags = _common_flags(abi, ext_name)
+    build_dir = CSRC / f".build{ext_name}"
     build_dir.mkdir(exist_ok=True)
     newest = max((CSRC / s).stat().st_mtime
-                 for s in LATENT_SOURCES + ["common.h"])
-    if (LATENT_SO_PATH.exists() and not force
-            and LATENT_SO_PATH.stat().st_mtime >= newest):
-        return LATENT_SO_PATH
+                 for s in sources + ["common.h"])
+    if (so_path.exists() and not force
+            and so_path.stat().st_mtime >= newest):
+        return so_path
     cmds, objs = [], []
-    for src in LATENT_SOURCES:
+    for src in sources:
         obj = build_dir / (Path(src).stem + ".o")
         cmd = ["hipcc", *flags, *inc_flags, "-c", str(CSRC / src), "-o", str(obj)]
         if src.endswith(".cpp"):
@@ -161,20 +181,24 @@ def build_latent(verbose: bool = False, force: bool = True) -> Path:
         if pr.returncode != 0:
             raise RuntimeError(f"build command failed ({' '.join(c[:3])} ...):"
                                f"\n{err[-8000:]}")
-    tmp = build_dir / f"_hip_latent.{os.getpid()}.so"
+    tmp = build_dir / f"{ext_name}.{os.getpid()}.so"
     _run(["hipcc", "-shared", f"--offload-arch={ARCH}", *objs, f"-L{libdir}",
           "-ltorch", "-ltorch_hip", "-ltorch_cpu", "-lc10", "-lc10_hip",
           "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
           f"-Wl,-rpath,{libdir}", "-o", str(tmp)])
-    os.replace(tmp, LATENT_SO_PATH)
-    return LATENT_SO_PATH
+    os.replace(tmp, so_path)
+    return so_path
 
 
 if __name__ == "__main__":
     if "--latent" in sys.argv:
         build_latent(verbose=True)
         print(f"built {LATENT_SO_PATH}")
+    elif "--paged" in sys.argv:
+        build_paged(verbose=True)
+        print(f"built {PAGED_SO_PATH}")
     else:
         build(verbose=True, force="--force" in sys.argv)
         build_latent(verbose=True)
-        print(f"built {SO_PATH} {LATENT_SO_PATH}")
+        build_paged(verbose=True)
+        print(f"built {SO_PATH} {LATENT_SO_PATH} {PAGED_SO_PATH}")

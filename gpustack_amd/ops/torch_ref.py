@@ -455,3 +455,134 @@ def moe_combine(out: torch.Tensor, y: torch.Tensor, inv: torch.Tensor,
 
 def softcap_(logits: torch.Tensor, cap: float) -> None:
     logits.copy_(cap * torch.tanh(logits / cap))
+
+
+# --- paged rotary attention family (ops/csrc/rowmix32.hip, ragged_attn.hip) --
+# fp32 stream with pre- and post-norms around every sublayer; rotary keys
+# in a paged pool with transposed value pages; scores, softmax and norms in
+# fp32 whatever the GEMM dtype.
+
+def embed_rows_f32(x: torch.Tensor, tokens: torch.Tensor,
+                   embed: torch.Tensor) -> None:
+    x.copy_(embed[tokens].float())
+
+
+def sandwich_add_norm(x: torch.Tensor, a: torch.Tensor | None,
+                      post_w: torch.Tensor | None, mult: float, eps: float,
+                      extra: torch.Tensor | None,
+                      next_w: torch.Tensor | None,
+                      h: torch.Tensor | None) -> None:
+    """x += mult * rmsnorm(a) * post_w  (+ extra), in fp32 on the fp32
+    stream x; then h = rmsnorm(x) * next_w in h's dtype. Either half may be
+    absent (a is None: no sublayer output; next_w is None: no next norm)."""
+    if a is not None:
+        af = a.float()
+        y = af * torch.rsqrt(af.pow(2).mean(-1, keepdim=True) + eps)
+        x.add_(y * post_w.float() * mult)
+    if extra is not None:
+        x.add_(extra.float())
+    if next_w is not None:
+        y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+        h.copy_((y * next_w.float()).to(h.dtype))
+
+
+def rotary_norm_store(q_out: torch.Tensor, qkv: torch.Tensor, nq: int,
+                      nk: int, q_norm_w: torch.Tensor | None,
+                      k_norm_w: torch.Tensor | None, inv_freq: torch.Tensor,
+                      pos32: torch.Tensor, head_dim: int,
+                      k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      slots: torch.Tensor, eps: float, tied: bool) -> None:
+    """Row kernel between the fused q/k/v projection and attention.
+    qkv[:, :nq] are the queries, [nq:nq+nk] the keys, the rest the values
+    (tied: none — the raw key projection serves as the value). Optionally a weighted
+    RMS norm over the WHOLE q and k rows, then pairwise rotary on the first
+    2*len(inv_freq) channels of every head_dim-wide head (angle = pos * f in
+    fp32). q goes to q_out [T, nq]; k to its slot of k_cache [nb, G, BS, KW];
+    v to its slot of the transposed pages v_cache [nb, G, VW, BS]."""
+    T = qkv.shape[0]
+    nb, G, BS, KW = k_cache.shape
+    VW = v_cache.shape[2]
+    q = qkv[:, :nq].float()
+    k = qkv[:, nq:nq + nk].float()
+    v = k if tied else qkv[:, nq + nk:].float()
+    if q_norm_w is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
+    half = inv_freq.numel()
+
+    def turn(t):
+        if half == 0:
+            return t
+        t = t.reshape(T, -1, head_dim).clone()
+        ang = pos32.to(torch.float32)[:, None] * inv_freq.float()[None, :]
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        u, w = t[..., 0:2 * half:2].clone(), t[..., 1:2 * half:2].clone()
+        t[..., 0:2 * half:2] = u * c - w * s
+        t[..., 1:2 * half:2] = w * c + u * s
+        return t.reshape(T, -1)
+
+    q_out.copy_(turn(q).to(q_out.dtype))
+    k = turn(k).to(k_cache.dtype).view(T, G, KW)
+    v = v.to(v_cache.dtype).view(T, G, VW)
+    ok = slots >= 0
+    blk, off = slots[ok] // BS, slots[ok] % BS
+    k_cache[blk, :, off] = k[ok]
+    v_cache[blk, :, :, off] = v[ok]
+
+
+def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
+                    v_cache: torch.Tensor, block_tables: torch.Tensor,
+                    row_seq: torch.Tensor, positions: torch.Tensor,
+                    scale: float, maps: int = 1, window: int = 0,
+                    keep_first: int = 0,
+                    sinks: torch.Tensor | None = None) -> None:
+    """out[t, a] = softmax_j(scale * q[t, a] . k_j) . V over the visible
+    keys j of row t's sequence: j <= pos(t), and with window > 0 also
+    (pos(t) - j < window or j < keep_first). q: [T, A, D] with A = heads *
+    maps score maps (a = head * maps + map); map m of a head reads channels
+    [m*D, (m+1)*D) of its kv head's key row and all maps weight the same
+    values. sinks (per head, or None) add exp(sink) to the denominator."""
+    T, A, D = q.shape
+    nb, G, BS, KW = k_cache.shape
+    VW = v_cache.shape[2]
+    H = A // maps
+    rep = H // G
+    for t in range(T):
+        p = int(positions[t])
+        bt = block_tables[int(row_seq[t])]
+        j = torch.arange(p + 1, device=q.device)
+        if window > 0:
+            j = j[(p - j < window) | (j < keep_first)]
+        blk = bt[j // BS].long()
+        K = k_cache[blk, :, j % BS].float()                  # [L, G, KW]
+        V = v_cache[blk, :, :, j % BS].float()               # [L, G, VW]
+        for a in range(A):
+            g = (a // maps) // rep
+            m = a % maps
+            s = (K[:, g, m * D:(m + 1) * D] @ q[t, a].float()) * scale
+            mx = s.max()
+            if sinks is not None:
+                mx = torch.maximum(mx, sinks[a // maps].float())
+            e = torch.exp(s - mx)
+            den = e.sum()
+            if sinks is not None:
+                den = den + torch.exp(sinks[a // maps].float() - mx)
+            out[t, a] = ((e / den) @ V[:, g]).to(out.dtype)
+
+
+def diff_combine(out: torch.Tensor, a: torch.Tensor, lam: torch.Tensor,
+                 diff: float, eps: float) -> None:
+    """a: [T, H, 2, VW] (two maps' outputs per head, fp32); out[t, h] =
+    unit_rms(a1 - lam * a2) * (1 - diff), RMS over the head's VW values."""
+    o = a[:, :, 0].float() - lam.float() * a[:, :, 1].float()
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * (1.0 - diff)
+    out.copy_(o.reshape(out.shape).to(out.dtype))
+
+
+def act_and_mul(out: torch.Tensor, gu: torch.Tensor, mode: str) -> None:
+    """out = act(gu[:, :F]) * gu[:, F:] (the gate in fp32 through the
+    activation, the product rounded once)."""
+    F_ = out.shape[1]
+    g = gu[:, :F_].float().clone()
+    act_inplace(g, mode)
+    out.copy_((g * gu[:, F_:].float()).to(out.dtype))
