@@ -24,9 +24,79 @@ class LatentMixerSpec:
 
 
 @dataclass(frozen=True)
+class RotarySpec:
+    """Pairwise rotary positions on the first `dims` channels of a head:
+    channel 2i pairs with 2i+1 and turns by pos * f_i, f_i = base^(-2i/dims),
+    optionally with wavelength-dependent frequency scaling (`scaling`:
+    factor / low / high / original — long waves slowed by `factor`, short
+    ones kept, a linear blend between)."""
+    dims: int = 0
+    base: float = 10000.0
+    scaling: tuple | None = None        # (factor, low, high, original)
+
+    def inv_freq(self) -> list[float]:
+        """f_i for i < dims/2, in double precision."""
+        import math
+
+        out = []
+        for i in range(self.dims // 2):
+            f = self.base ** (-2.0 * i / self.dims)
+            if self.scaling is not None:
+                factor, low, high, orig = self.scaling
+                wave = 2.0 * math.pi / f
+                if wave > orig / low:
+                    f = f / factor
+                elif wave >= orig / high:
+                    s = (orig / wave - low) / (high - low)
+                    f = (1.0 - s) * f / factor + s * f
+            out.append(f)
+        return out
+
+
+@dataclass(frozen=True)
+class PagedMixerSpec:
+    """Rotary softmax attention over a paged key/value pool
+    (models/paged_attention.py). Every option is a parameter:
+
+    * maps = 2: differential attention — q and k carry two score maps per
+      head (a head's two maps adjacent, heads in order), both weight the same values, and
+      the head's output is a1 - lambda * a2, unit-RMS-normalised and scaled
+      by (1 - diff); lambda = exp(lq1.lk1) - exp(lq2.lk2) + diff.
+    * window > 0: a row sees keys closer than `window` plus the first
+      `keep_first` keys of its sequence, whose positions stay what they are.
+    * sink: one learned logit per head joins the softmax denominator.
+    * qk_norm_full: weighted RMS norm over the whole q (and k) projection,
+      before rotation.
+    * tied_values: no value projection of its own; the raw key projection
+      (neither normed nor rotated) serves as the value."""
+    heads: int
+    kv_heads: int
+    qk_dim: int
+    v_dim: int
+    scale: float
+    rot: RotarySpec = RotarySpec()
+    bias: bool = False
+    maps: int = 1
+    diff: float = 0.0
+    window: int = 0
+    keep_first: int = 0
+    sink: bool = False
+    qk_norm_full: bool = False
+    tied_values: bool = False
+
+    @property
+    def k_width(self) -> int:           # cached key channels per kv head
+        return self.maps * self.qk_dim
+
+    @property
+    def v_width(self) -> int:
+        return self.qk_dim if self.tied_values else self.v_dim
+
+
+@dataclass(frozen=True)
 class FeedForwardSpec:
-    """Ungated feed-forward W_down act(W_up h), dense or as a bank of
-    routed experts (models/experts.py). Routing: softmax scores over all
+    """Feed-forward W_down act(W_up h) — with `gated`, W_down (act(W_gate h)
+    * W_up h) — dense or as a bank of routed experts (models/experts.py). Routing: softmax scores over all
     experts, group-limited top-k (groups of neighbouring experts ranked by
     their best member, keep_groups stay eligible), weights = score *
     route_scale without renormalisation; shared_ff > 0 adds an always-on
@@ -41,13 +111,14 @@ class FeedForwardSpec:
     route_scale: float = 1.0
     shared_ff: int = 0
     shared_gated: bool = False
+    gated: bool = False
 
 
 @dataclass(frozen=True)
 class LayerSpec:
     """One entry of a heterogeneous layer stack (ModelSpec.layers)."""
-    mixer_type: str
-    mixer: LatentMixerSpec
+    mixer_type: str                      # "latent_attention" | "paged_attention"
+    mixer: "LatentMixerSpec | PagedMixerSpec"
     mlp: FeedForwardSpec | None = None
 
 
@@ -167,14 +238,45 @@ class ModelSpec:
     bigram_buckets: int = 0
     bigram_mul_prev: int = 0
     bigram_mul_cur: int = 0
+    # weight-shared loop over a span of a heterogeneous stack: layers
+    # start..stop-1 run `times` times in a row with the same weights, every
+    # pass with cache pools of its own; each pass but the first starts by
+    # adding the embedding output to the stream. None = every layer once
+    layer_loop: tuple | None = None      # (start, stop, times)
 
     @property
     def gqa_ratio(self) -> int:
         return self.num_heads // self.num_kv_heads
 
+    def layer_runs(self) -> list[tuple[int, bool]]:
+        """Execution order of a heterogeneous stack: one (layer index,
+        re-inject the embedding first) entry per layer RUN. A looped layer
+        appears once per pass; cache pools are per run, weights per layer."""
+        n = len(self.layers)
+        if not self.layer_loop:
+            return [(i, False) for i in range(n)]
+        start, stop, times = self.layer_loop
+        runs = [(i, False) for i in range(start)]
+        for t in range(times):
+            runs += [(i, t > 0 and i == start) for i in range(start, stop)]
+        return runs + [(i, False) for i in range(stop, n)]
+
+    def kv_pool_widths(self) -> list[tuple]:
+        """Per layer run of a heterogeneous stack: ("latent", rank) or
+        ("kv", kv_heads, key width, value width)."""
+        out = []
+        for i, _ in self.layer_runs():
+            m = self.layers[i].mixer
+            if isinstance(m, LatentMixerSpec):
+                out.append(("latent", m.kv_rank))
+            else:
+                out.append(("kv", m.kv_heads, m.k_width, m.v_width))
+        return out
+
     def kv_bytes_per_token(self, dtype_size: int = 2) -> int:
         if self.layers is not None:
-            return sum(ls.mixer.kv_rank for ls in self.layers) * dtype_size
+            return sum(w[1] if w[0] == "latent" else w[1] * (w[2] + w[3])
+                       for w in self.kv_pool_widths()) * dtype_size
         if self.kv_lora_rank:
             # MLA: one compressed latent row per token per layer
             return (self.num_layers
@@ -190,6 +292,14 @@ class ModelSpec:
                 n += (self.bigram_buckets + 1) * h
             for ls in self.layers:
                 m = ls.mixer
+                if isinstance(m, PagedMixerSpec):
+                    n += (h * m.maps * m.qk_dim * (m.heads + m.kv_heads)
+                          + (0 if m.tied_values else h * m.kv_heads * m.v_dim)
+                          + m.heads * m.v_dim * h + 4 * h)
+                    f = ls.mlp
+                    if f is not None:
+                        n += (3 if f.gated else 2) * h * f.ff
+                    continue
                 n += (h * m.heads * m.qk_dim + h * m.kv_rank + m.kv_rank
                       + m.kv_rank * m.heads * (m.qk_dim + m.v_dim)
                       + m.heads * m.v_dim * h + 2 * h)
@@ -306,9 +416,85 @@ class ModelSpec:
         )
 
     @classmethod
+    def _from_fusipel_config(cls, cfg: dict) -> "ModelSpec":
+        """Fusipel checkpoints list their layers like Vunitar ones: every
+        entry names its mixer — "attention" (two-map differential scores,
+        sliding window with kept first keys, own value projection) or
+        "attention_2" (whole-projection q/k norm, values tied to the keys,
+        per-head sink) — with its sizes and constants, and an optional
+        gated dense feed-forward. `loop` repeats a span of the stack."""
+        def rotary(r):
+            if not r or not int(r.get("dims", 0) or 0):
+                return RotarySpec()
+            sc = r.get("scaling") or None
+            return RotarySpec(
+                dims=int(r["dims"]), base=float(r["base"]),
+                scaling=(float(sc["factor"]), float(sc["low"]),
+                         float(sc["high"]), float(sc["original"]))
+                if sc else None)
+
+        layers = []
+        for ent in cfg["layers"]:
+            m = ent["mixer"]
+            common = dict(
+                heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                qk_dim=int(m["dim"]), v_dim=int(m.get("vdim", m["dim"])),
+                scale=float(m["scale"]), rot=rotary(m.get("rot")), bias=True)
+            if ent["type"] == "attention":
+                mask = m.get("mask") or {}
+                mixer = PagedMixerSpec(
+                    **common, maps=2, diff=float(m["diff"]),
+                    window=int(mask.get("size", 0) or 0),
+                    keep_first=int(mask.get("keep_first", 0) or 0))
+            elif ent["type"] == "attention_2":
+                mixer = PagedMixerSpec(
+                    **common, sink=True, qk_norm_full=True, tied_values=True)
+            else:
+                raise NotImplementedError(
+                    f"Fusipel mixer type {ent['type']!r} is not implemented")
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+            if mixer.rot.dims % 2 or mixer.rot.dims > mixer.qk_dim:
+                raise ValueError("rotary dims must be even and fit the head")
+            f = ent.get("mlp")
+            if not f:
+                ff = None
+            elif f["kind"] == "dense":
+                ff = FeedForwardSpec(kind="dense", ff=int(f["ff"]),
+                                     act="gelu_tanh", gated=True)
+            else:
+                raise NotImplementedError(
+                    f"Fusipel feed-forward kind {f['kind']!r}")
+            layers.append(LayerSpec("paged_attention", mixer, ff))
+        loop = cfg.get("loop") or None
+        if loop:
+            start, stop, times = (int(loop["start"]), int(loop["stop"]),
+                                  int(loop["times"]))
+            if not (0 <= start <= stop <= len(layers)) or times < 1:
+                raise ValueError("loop span outside the layer list")
+            loop = (start, stop, times) if stop > start else None
+        return cls(
+            architecture="Fusipel",
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            num_layers=len(layers),
+            layers=tuple(layers),
+            layer_loop=loop,
+            num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+            rms_norm_eps=float(cfg["norm"]["eps"]),
+            max_position_embeddings=int(
+                cfg.get("max_position_embeddings", 1 << 20)),
+            eos_token_id=int(cfg.get("eos_token_id", -1)),
+            sandwich_norms=True, fp32_residual=True,
+            residual_multiplier=float(cfg.get("residual_mult", 1.0)),
+        )
+
+    @classmethod
     def from_hf_config(cls, cfg: dict) -> "ModelSpec":
         if cfg.get("architecture") == "Vunitar" and "architectures" not in cfg:
             return cls._from_vunitar_config(cfg)
+        if cfg.get("architecture") == "Fusipel" and "architectures" not in cfg:
+            return cls._from_fusipel_config(cfg)
         arch = (cfg.get("architectures") or ["LlamaForCausalLM"])[0]
         if arch.startswith("Cohere") and cfg.get("use_qk_norm"):
             raise NotImplementedError(

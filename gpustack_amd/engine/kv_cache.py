@@ -176,18 +176,37 @@ class KVCache:
             dtype = getattr(torch, cfg.dtype)
         self.kv_dtype = dtype
         if self.layered:
-            self.k_caches = [
-                torch.zeros((num_blocks, self.latent_planes(cfg),
-                             cfg.block_size, ls.mixer.kv_rank),
-                            dtype=dtype, device=device)
-                for ls in spec.layers[:self.num_layers]
-            ]
+            # one pool (pair) per layer RUN: a weight-shared loop gives
+            # every pass its own. Paged-attention runs keep keys as
+            # [nblocks, kv_heads, BS, key width] (rotated, all score maps of
+            # a head side by side) and values with every page transposed,
+            # [nblocks, kv_heads, value width, BS], so that both matrix
+            # products of ops.paged_attention find their reduction axis
+            # contiguous (scores reduce over channels, the weighted sum
+            # over keys)
+            widths = spec.kv_pool_widths()
+            self.num_layers = len(widths)
+            self.k_caches, self.v_caches = [], []
+            for w in widths:
+                if w[0] == "latent":
+                    ks = (num_blocks, self.latent_planes(cfg), cfg.block_size,
+                          w[1])
+                    vs = (0,)
+                else:
+                    ks = (num_blocks, w[1], cfg.block_size, w[2])
+                    vs = (num_blocks, w[1], w[3], cfg.block_size)
+                self.k_caches.append(torch.zeros(ks, dtype=dtype,
+                                                 device=device))
+                self.v_caches.append(torch.zeros(vs, dtype=dtype,
+                                                 device=device))
         else:
             self.k_caches = [
                 torch.zeros(shape, dtype=dtype, device=device)
                 for _ in range(self.num_layers)
             ]
-        if self.mla:
+        if self.layered:
+            pass
+        elif self.mla:
             self.v_caches = [
                 torch.zeros(0, dtype=dtype, device=device)
                 for _ in range(self.num_layers)
@@ -294,8 +313,10 @@ class KVCache:
         esize = 1 if cfg.kv_cache_dtype == "fp8" else 2
         if spec.layers is not None:
             esize = 4 if cfg.dtype == "float32" else 2
-            per_block = (cfg.block_size * spec.kv_bytes_per_token(esize)
-                         * KVCache.latent_planes(cfg))
+            planes = KVCache.latent_planes(cfg)
+            per_block = cfg.block_size * esize * sum(
+                w[1] * planes if w[0] == "latent" else w[1] * (w[2] + w[3])
+                for w in spec.kv_pool_widths())
         elif spec.kv_lora_rank:
             per_block = (nl * cfg.block_size
                          * (spec.kv_lora_rank + spec.qk_rope_head_dim)

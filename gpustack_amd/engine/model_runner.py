@@ -269,6 +269,8 @@ class ModelRunner:
             load_safetensors(self.model, cfg, cfg.model_dir)
         else:
             random_init(self.model, cfg)
+        if hasattr(self.model, "post_load"):
+            self.model.post_load()   # constants derived from the weights
         if cfg.lora_dirs:
             from ..models.weights import merge_lora
 

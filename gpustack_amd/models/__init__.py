@@ -4,6 +4,7 @@ from .llama import LlamaForCausalLM
 # runs on the flag-driven llama-lineage graph.
 _MODEL_CLASSES = {
     "Vunitar": ("vunitar", "VunitarForCausalLM"),
+    "Fusipel": ("fusipel", "FusipelForCausalLM"),
 }
 
 

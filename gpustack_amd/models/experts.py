@@ -1,7 +1,10 @@
-"""Ungated feed-forward blocks: dense, and a routed expert bank.
+"""Feed-forward blocks of the layer-listed models: dense, and a routed
+expert bank.
 
-Both compute W_down act(W_up h) with a selectable activation (the gated
-SiLU blocks of the llama lineage live in models/llama.py). The bank routes
+Both compute W_down act(W_up h) with a selectable activation; the dense
+block also has a gated form, W_down (act(W_gate h) * W_up h), with gate and
+up fused into one GEMM (the gated SiLU blocks of the llama lineage live in
+models/llama.py). The bank routes
 with full-softmax scores and group-limited top-k — experts sit in equal
 groups of neighbours, a group is ranked by its best member, only the best
 `keep_groups` groups stay eligible — and weights the chosen experts by
@@ -26,15 +29,23 @@ class DenseFF(nn.Module):
         super().__init__()
         if comm is not None and comm.tp_size > 1:
             raise NotImplementedError("ungated FF is not TP-sharded yet")
-        self.act = f.act
-        self.up_w = nn.Parameter(torch.empty(f.ff, width, dtype=dtype),
-                                 requires_grad=False)
+        self.act, self.gated, self.ff = f.act, f.gated, f.ff
+        # gated: rows [0, ff) are the gate, [ff, 2 ff) the up projection
+        self.up_w = nn.Parameter(
+            torch.empty(f.ff * (2 if f.gated else 1), width, dtype=dtype),
+            requires_grad=False)
         self.down_w = nn.Parameter(torch.empty(width, f.ff, dtype=dtype),
                                    requires_grad=False)
 
-    def forward(self, h, x32):
+    def forward(self, h, x32=None):
         u = F.linear(h, self.up_w)
-        ops.act_inplace(u, self.act)
+        if self.gated:
+            g = torch.empty(h.shape[0], self.ff, dtype=h.dtype,
+                            device=h.device)
+            ops.act_and_mul(g, u, self.act)
+            u = g
+        else:
+            ops.act_inplace(u, self.act)
         return F.linear(u, self.down_w)
 
 

@@ -55,6 +55,36 @@ class RaggedMeta:
             self._tiles[heads] = t
         return t
 
+    def page_groups(self, block_size: int):
+        """Runs of rows inside one cache page (ops.build_page_groups), or
+        None for a batch of single rows, whose values go row by row."""
+        if max(self.seq_news, default=1) <= 1:
+            return None
+        if self._tiles is None:
+            self._tiles = {}
+        key = ("pages", block_size)
+        g = self._tiles.get(key)
+        if g is None:
+            g = ops.build_page_groups(self.seq_starts, self.seq_hists,
+                                      self.seq_news, block_size,
+                                      self.block_tables.device)
+            self._tiles[key] = g
+        return g
+
+    def attn_tiles(self, heads: int, kv_heads: int, maps: int):
+        """Workgroup tile list for ops.paged_attention, cached per head
+        layout (layers of one model may differ in it)."""
+        if self._tiles is None:
+            self._tiles = {}
+        key = (heads, kv_heads, maps)
+        t = self._tiles.get(key)
+        if t is None:
+            t = ops.build_attn_tiles(self.seq_starts, self.seq_hists,
+                                     self.seq_news, heads, kv_heads, maps,
+                                     self.block_tables.device)
+            self._tiles[key] = t
+        return t
+
 
 @dataclass
 class ForwardMeta:

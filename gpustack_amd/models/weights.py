@@ -57,13 +57,16 @@ def _layered_tensor_plan(model):
     plan = []
     same = lambda t: t
     plan.append(("embed", model.embed, same))
-    if model.pair_table is not None:
+    if getattr(model, "pair_table", None) is not None:
         plan.append(("bigram", model.pair_table, same))
     plan.append(("final.norm", model.final_norm, same))
     plan.append(("head", model.lm_head, same))
     for i, layer in enumerate(model.layers):
         p = f"l{i}."
         a = layer.attn
+        if hasattr(a, "qkv_w"):
+            plan += _paged_layer_plan(p, layer)
+            continue
         nq = a.h * a.dq
         plan += [
             (p + "mix.q", a.qd_w[:nq], same),
@@ -96,15 +99,61 @@ def _layered_tensor_plan(model):
     return plan
 
 
+def _paged_layer_plan(p: str, layer):
+    """Plan entries of one pre/post-norm layer with a paged rotary mixer
+    (models/paged_attention.py) and an optional gated dense feed-forward:
+    q, k (and v) with their biases fuse into one projection, gate and up
+    into another; norm weights, sinks and the lambda vectors stay fp32."""
+    same = lambda t: t
+    a = layer.attn
+    nq, nk, nv = a.nq, a.nk, a.nv
+    plan = [
+        (p + "norm1", layer.pre1, same), (p + "norm1b", layer.post1, same),
+        (p + "mix.q", a.qkv_w[:nq], same),
+        (p + "mix.k", a.qkv_w[nq:nq + nk], same),
+        (p + "mix.o", a.o_w, same),
+    ]
+    if a.qkv_b is not None:
+        plan += [(p + "mix.q.b", a.qkv_b[:nq], same),
+                 (p + "mix.k.b", a.qkv_b[nq:nq + nk], same)]
+    if nv:
+        plan.append((p + "mix.v", a.qkv_w[nq + nk:], same))
+        if a.qkv_b is not None:
+            plan.append((p + "mix.v.b", a.qkv_b[nq + nk:], same))
+    if a.q_norm is not None:
+        plan += [(p + "mix.q.norm", a.q_norm, same),
+                 (p + "mix.k.norm", a.k_norm, same)]
+    if a.sinks is not None:
+        plan.append((p + "mix.sink", a.sinks, same))
+    if a.lam_vecs is not None:
+        plan += [(p + f"mix.{n}", a.lam_vecs[j], same)
+                 for j, n in enumerate(("lq1", "lk1", "lq2", "lk2"))]
+    m = layer.mlp
+    if m is not None:
+        plan += [(p + "norm2", layer.pre2, same),
+                 (p + "norm2b", layer.post2, same),
+                 (p + "mlp.down", m.down_w, same)]
+        if m.gated:
+            plan += [(p + "mlp.gate", m.up_w[:m.ff], same),
+                     (p + "mlp.up", m.up_w[m.ff:], same)]
+        else:
+            plan.append((p + "mlp.up", m.up_w, same))
+    return plan
+
+
 def _random_init_layered(model, cfg: EngineConfig) -> None:
     """Random weights for a heterogeneous-stack model: projections N(0,
     1/fan_in), norm and layer-scale weights near 1 / near 0.5, so deep
     random stacks keep O(1) activations."""
     for name, dst, fn in _layered_tensor_plan(model):
         if dst.dim() == 1 and not name.endswith(("router", "sg")):
-            base = 0.5 if name.rsplit(".", 1)[-1] in ("ls1", "ls2") else 1.0
+            leaf = name.rsplit(".", 1)[-1]
+            if leaf in ("b", "sink", "lq1", "lk1", "lq2", "lk2"):
+                base, std = 0.0, 0.3     # biases, sinks, lambda vectors
+            else:
+                base, std = (0.5 if leaf in ("ls1", "ls2") else 1.0), 0.05
             t = base + _gen(tuple(dst.shape), name, cfg.seed, torch.float32,
-                            model.device, std=0.05)
+                            model.device, std=std)
             dst.copy_(t.to(dst.dtype))
             continue
         # generate in the checkpoint's own [out, in] shape, then apply the
