@@ -56,10 +56,14 @@ def parse_args():
                     help="prefill-context-parallel degree (rows chunked "
                          "across ranks, replicated decode); world = tp*cp")
     ap.add_argument("--layer-bench", action="store_true",
-                    help="instead of the serving workload: Vunitar layers at "
+                    help="instead of the serving workload: Vunitar or Fusipel "
+                         "layers (--layer-family) at "
                          "real-model sizes beside the closest llama-lineage "
                          "stack (prefill/decode tok/s + per-kernel roofline "
                          "shares; gpustack_amd/bench/layer_bench.py)")
+    ap.add_argument("--layer-family", default="vunitar",
+                    choices=["vunitar", "fusipel"],
+                    help="model family measured by --layer-bench")
     ap.add_argument("--layer-sizes", default="small,medium",
                     help="comma list of small,medium,large for --layer-bench")
     return ap.parse_args()
@@ -72,7 +76,8 @@ def main():
 
         run_layer_bench(args.layer_sizes.split(","),
                         args.device or ("cuda:0" if torch.cuda.is_available()
-                                        else "cpu"))
+                                        else "cpu"),
+                        family=args.layer_family)
         return
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

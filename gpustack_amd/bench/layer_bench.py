@@ -1,12 +1,12 @@
-"""Layer-level comparison bench: a Vunitar stack at real-model layer sizes
-beside the closest llama-lineage stack of equal width, depth and heads
-(random weights, synthetic tokens). Reports end-to-end prefill and decode
+"""Layer-level comparison bench: a Vunitar or Fusipel stack (`family`) at
+real-model layer sizes beside the closest llama-lineage stack of equal
+width, depth and heads (random weights, synthetic tokens). Reports end-to-end prefill and decode
 throughput through LLMEngine for both, and per-kernel rates of the new
 kernels next to their counterparts with the fraction of the MI355X
 roofline each reaches (2.5 PFLOP/s dense bf16, 8 TB/s HBM3E).
 
-Run through `python bench.py --layer-bench [--layer-sizes small,medium]`;
-bench.py's default workload is untouched.
+Run through `python bench.py --layer-bench [--layer-family fusipel]
+[--layer-sizes small,medium]`; bench.py's default workload is untouched.
 """
 from __future__ import annotations
 
@@ -49,6 +49,34 @@ def vunitar_spec(s, moe: bool):
         norm_after=True, layer_scale=True, fp32_residual=True,
         final_logit_softcap=30.0, bigram_buckets=4093, bigram_mul_prev=131,
         bigram_mul_cur=17)
+
+
+def fusipel_spec(s, moe: bool = False):
+    """Alternating mixers at head size 128: values tied to the keys with a
+    sink (heads/4 kv heads), and two-map differential attention behind a
+    512-key window that keeps 4 first keys (half the heads, two maps each);
+    gated tanh-GELU feed-forward of the llama stack's width."""
+    from ..engine.config import (FeedForwardSpec, LayerSpec, ModelSpec,
+                                 PagedMixerSpec, RotarySpec)
+
+    H = s["heads"]
+    rot = RotarySpec(dims=64, base=10000.0, scaling=(8.0, 1.0, 4.0, 8192.0))
+    tied = PagedMixerSpec(heads=H, kv_heads=max(1, H // 4), qk_dim=128,
+                          v_dim=128, scale=128 ** -0.5, rot=rot, bias=True,
+                          sink=True, qk_norm_full=True, tied_values=True)
+    diff = PagedMixerSpec(heads=max(1, H // 2), kv_heads=max(1, H // 8),
+                          qk_dim=128, v_dim=128, scale=128 ** -0.5, rot=rot,
+                          bias=True, maps=2, diff=0.4, window=512,
+                          keep_first=4)
+    ff = FeedForwardSpec(kind="dense", ff=s["ff"], act="gelu_tanh", gated=True)
+    return ModelSpec(
+        architecture="Fusipel", vocab_size=32000, hidden_size=s["width"],
+        num_layers=s["layers"],
+        layers=tuple(LayerSpec("paged_attention", diff if i % 2 else tied, ff)
+                     for i in range(s["layers"])),
+        num_heads=1, num_kv_heads=1, head_dim=8, intermediate_size=0,
+        rms_norm_eps=1e-6, max_position_embeddings=1 << 20, eos_token_id=-1,
+        sandwich_norms=True, fp32_residual=True, residual_multiplier=0.7)
 
 
 def llama_spec(s, moe: bool):
@@ -247,15 +275,173 @@ def kernel_rates(s, device):
     return out
 
 
-def run(sizes: list[str], device: str) -> None:
+def fusipel_kernel_rates(s, device):
+    """Per-kernel rates of the paged rotary attention family next to the
+    llama graph's counterparts."""
+    from .. import ops
+
+    bf = torch.bfloat16
+    H, W, D, BS = s["heads"], s["width"], 128, 16
+    G = max(1, H // 4)
+    out = []
+
+    def rec(name, sec, flops=None, nbytes=None):
+        if flops is not None:
+            out.append(dict(kernel=name, us=round(sec * 1e6, 1),
+                            tflops=round(flops / sec / 1e12, 1),
+                            roofline=round(flops / sec / PEAK_FLOPS, 4)))
+        else:
+            out.append(dict(kernel=name, us=round(sec * 1e6, 1),
+                            gbps=round(nbytes / sec / 1e9, 1),
+                            roofline=round(nbytes / sec / PEAK_BW, 4)))
+
+    def pools(nblk, g, kw, vw):
+        return (torch.randn(nblk, g, BS, kw, device=device).to(bf),
+                torch.randn(nblk, g, vw, BS, device=device).to(bf))
+
+    # ---- prefill attention: 4 prompts x 2048 ----
+    nseq, L = 4, 2048
+    T = nseq * L
+    pairs = nseq * L * (L + 1) // 2
+    nblk = T // BS + 1
+    bt = torch.arange(nseq * (L // BS), dtype=torch.int32, device=device).view(nseq, -1)
+    row_seq = torch.arange(nseq, dtype=torch.int32, device=device).repeat_interleave(L)
+    pos = torch.arange(L, dtype=torch.int32, device=device).repeat(nseq)
+    starts = [i * L for i in range(nseq)]
+    kc, vc = pools(nblk, G, D, D)
+    q = torch.randn(T, H, D, device=device).to(bf)
+    o = torch.empty_like(q)
+    sinks = torch.zeros(H, device=device)
+    tiles = ops.build_attn_tiles(starts, [0] * nseq, [L] * nseq, H, G, 1, device)
+    rec("paged_attention prefill, causal + sink (mfma)",
+        _time(lambda: ops.paged_attention(o, q, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, sinks=sinks, tiles=tiles), 5),
+        flops=4.0 * D * H * pairs)
+    # two maps, window 512 + 4 kept: H/2 heads x 2 maps = H score maps
+    Gd = max(1, H // 8)
+    kc2, vc2 = pools(nblk, Gd, 2 * D, D)
+    o32 = torch.empty(T, H, D, device=device)
+    tiles2 = ops.build_attn_tiles(starts, [0] * nseq, [L] * nseq,
+                                  max(1, H // 2), Gd, 2, device)
+    wpairs = nseq * sum(min(i + 1, 512 + 4) for i in range(L))
+    rec("paged_attention prefill, 2 maps, window 512 (mfma)",
+        _time(lambda: ops.paged_attention(o32, q, kc2, vc2, bt, row_seq, pos,
+                                          D ** -0.5, maps=2, window=512,
+                                          keep_first=4, tiles=tiles2), 5),
+        flops=4.0 * D * H * wpairs)
+    kf = torch.randn(T, G, D, device=device).to(bf)
+    vf = torch.randn_like(kf)
+    of = torch.empty_like(q)
+    ptiles = ops.build_prefill_tiles([L] * nseq, device)
+    rec("flash_prefill (llama graph)",
+        _time(lambda: ops.varlen_prefill_attn(of, q, kf, vf, [L] * nseq,
+                                              D ** -0.5, tiles=ptiles), 5),
+        flops=4.0 * D * H * pairs)
+
+    # ---- decode attention: 64 sequences x 2048 cached ----
+    B, Lc = 64, 2048
+    nblk = B * (Lc // BS) + 1
+    bt = torch.arange(B * (Lc // BS), dtype=torch.int32, device=device).view(B, -1)
+    row_seq = torch.arange(B, dtype=torch.int32, device=device)
+    pos = torch.full((B,), Lc - 1, dtype=torch.int32, device=device)
+    kc, vc = pools(nblk, G, D, D)
+    qd = torch.randn(B, H, D, device=device).to(bf)
+    od = torch.empty_like(qd)
+    tiles = ops.build_attn_tiles(list(range(B)), [Lc - 1] * B, [1] * B, H, G, 1,
+                                 device)
+    rec("paged_attention decode, causal + sink (mfma)",
+        _time(lambda: ops.paged_attention(od, qd, kc, vc, bt, row_seq, pos,
+                                          D ** -0.5, sinks=sinks, tiles=tiles,
+                                          max_ctx=Lc)),
+        nbytes=B * Lc * G * D * 2 * 2)
+    kl = torch.randn(nblk, G, BS, D, device=device).to(bf)
+    vl = torch.randn_like(kl)
+    lens = torch.full((B,), Lc, dtype=torch.int32, device=device)
+    rec("paged_attn_decode (llama graph)",
+        _time(lambda: ops.paged_attn_decode(od, qd, kl, vl, bt, lens, D ** -0.5)),
+        nbytes=B * Lc * G * D * 2 * 2)
+
+    # ---- row kernels at T = 8192 ----
+    T = 8192
+    x = torch.randn(T, W, device=device)
+    a = torch.randn(T, W, device=device).to(bf)
+    w32 = torch.ones(W, device=device)
+    hb = torch.empty(T, W, dtype=bf, device=device)
+    rec("sandwich_add_norm (post-norm + add + pre-norm, fp32 stream)",
+        _time(lambda: ops.sandwich_add_norm(x, a, w32, 0.5, 1e-6, None, w32, hb)),
+        nbytes=T * W * 12)
+    xb, rb = a.clone(), a.clone()
+    wb = torch.ones(W, dtype=bf, device=device)
+    rec("fused_add_rms_norm (llama graph)",
+        _time(lambda: ops.fused_add_rms_norm(xb, rb, wb, 1e-6)),
+        nbytes=T * W * 8)
+    gu = torch.randn(T, 2 * s["ff"], device=device).to(bf)
+    ao = torch.empty(T, s["ff"], dtype=bf, device=device)
+    rec("act_and_mul gelu_tanh", _time(lambda: ops.act_and_mul(ao, gu, "gelu_tanh")),
+        nbytes=T * s["ff"] * 6)
+    rec("silu_and_mul (llama graph)", _time(lambda: ops.silu_and_mul(ao, gu)),
+        nbytes=T * s["ff"] * 6)
+    nblk = T // BS + 1
+    nq, nk = H * D, G * D
+    kc, vc = pools(nblk, G, D, D)
+    qkv = torch.randn(T, nq + nk, device=device).to(bf)
+    qo = torch.empty(T, nq, dtype=bf, device=device)
+    qw, kw = torch.ones(nq, device=device), torch.ones(nk, device=device)
+    inv = torch.tensor([10000.0 ** (-i / 32) for i in range(32)], device=device)
+    slots = torch.arange(T, device=device)
+    p32 = torch.arange(T, dtype=torch.int32, device=device)
+    rec("rotary_norm_store, values row by row (decode's way)",
+        _time(lambda: ops.rotary_norm_store(qo, qkv, nq, nk, qw, kw, inv, p32, D,
+                                            kc, vc, slots, 1e-6, True)),
+        nbytes=T * (2 * nq + 3 * nk) * 2)
+    pg = ops.build_page_groups([0], [0], [T], BS, device)
+    rec("rotary_norm_store (q/k norm + rotary + cache write, values by page)",
+        _time(lambda: ops.rotary_norm_store(qo, qkv, nq, nk, qw, kw, inv, p32, D,
+                                            kc, vc, slots, 1e-6, True,
+                                            page_groups=pg)),
+        nbytes=T * (2 * nq + 3 * nk) * 2)
+    kk = torch.randn(T, G, D, device=device).to(bf)
+    kl = torch.zeros(nblk, G, BS, D, dtype=bf, device=device)
+    vl = torch.zeros_like(kl)
+    rec("reshape_and_cache (llama graph)",
+        _time(lambda: ops.reshape_and_cache(kk, kk, kl, vl, slots)),
+        nbytes=T * G * D * 8)
+    # the same function as the llama graph runs it (its q/k-normed models):
+    # per-head norm of q, of k, rotary, cache write — four launches; priced
+    # with the fused kernel's byte count, so the shares compare times
+    qh = torch.randn(T, H, D, device=device).to(bf)
+    wn = torch.ones(D, dtype=bf, device=device)
+    cs = ops.build_cos_sin_cache(D, 64, T, 10000.0, None, device)
+    p64 = torch.arange(T, device=device)
+
+    def llama_chain():
+        ops.rms_norm(qh.view(-1, D), qh.view(-1, D), wn, 1e-6)
+        ops.rms_norm(kk.view(-1, D), kk.view(-1, D), wn, 1e-6)
+        ops.rotary_embedding(p64, qh, kk, cs, D, 64)
+        ops.reshape_and_cache(kk, kk, kl, vl, slots)
+
+    rec("rms_norm q, k + rotary_embedding + reshape_and_cache (llama graph)",
+        _time(llama_chain), nbytes=T * (2 * nq + 3 * nk) * 2)
+    a4 = torch.randn(T, max(1, H // 2), 2, D, device=device)
+    oc = torch.empty(T, max(1, H // 2) * D, dtype=bf, device=device)
+    lam = torch.tensor([0.7], device=device)
+    rec("diff_combine (a1 - lambda a2, unit rms)",
+        _time(lambda: ops.diff_combine(oc, a4, lam, 0.4, 1e-6)),
+        nbytes=T * H * D * 4 + T * (H // 2) * D * 2)
+    return out
+
+
+def run(sizes: list[str], device: str, family: str = "vunitar") -> None:
     for name in sizes:
         s = SIZES[name]
-        for moe in (False, True):
+        for moe in ((False, True) if family == "vunitar" else (False,)):
             row = {"size": name, **s, "ff_kind": "moe" if moe else "dense"}
-            for label, mk in (("vunitar", vunitar_spec), ("llama_graph", llama_spec)):
+            mine = vunitar_spec if family == "vunitar" else fusipel_spec
+            for label, mk in ((family, mine), ("llama_graph", llama_spec)):
                 pre, dec = engine_rates(mk(s, moe), device)
                 row[label] = {"prefill_tok_s": round(pre), "decode_tok_s": round(dec)}
             print(json.dumps({"layer_bench": row}), flush=True)
         if torch.cuda.is_available():
-            for k in kernel_rates(s, device):
+            rates = kernel_rates if family == "vunitar" else fusipel_kernel_rates
+            for k in rates(s, device):
                 print(json.dumps({"kernel_bench": {"size": name, **k}}), flush=True)
