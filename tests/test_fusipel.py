@@ -127,6 +127,65 @@ def test_rotary_frequencies(rot):
 
 # ---- each mechanism alone -----------------------------------------------------
 
+def test_rotation_and_whole_row_norm_alone():
+    """ops.rotary_norm_store against the oracle's pair rotation and unit
+    RMS: partial rotation, scaled frequencies, positions in the thousands."""
+    from gpustack_amd import ops
+
+    T, H, G, d, eps = 9, 3, 1, 10, 1e-5
+    rot = oracle.rot(6, base=30.0)
+    g = torch.Generator().manual_seed(4)
+    qkv = torch.randn(T, (H + G) * d, generator=g)
+    qw, kw = torch.rand(H * d, generator=g) + 0.5, torch.rand(G * d, generator=g) + 0.5
+    pos = torch.tensor([0, 1, 2, 17, 100, 999, 1000, 2047, 5000], dtype=torch.int32)
+    inv = torch.tensor(RotarySpec(dims=6, base=30.0, scaling=(3.0, 1.0, 3.0, 40.0)
+                                  ).inv_freq(), dtype=torch.float64).float()
+    kc = torch.zeros(T, G, 16, d)
+    vc = torch.zeros(T, G, d, 16)
+    slots = torch.arange(T) * 16 + 3
+    q = torch.empty(T, H * d)
+    ops.rotary_norm_store(q, qkv, H * d, G * d, qw, kw, inv, pos, d, kc, vc,
+                          slots, eps, True)
+    x = qkv.double()
+    rq = oracle.rotate_pairs(oracle.unit_rms(x[:, :H * d], eps, qw.double())
+                             .view(T, H, d), rot, pos)
+    rk = oracle.rotate_pairs(oracle.unit_rms(x[:, H * d:], eps, kw.double())
+                             .view(T, G, d), rot, pos)
+    assert (q.double().view(T, H, d) - rq).abs().max() < 1e-5
+    assert (kc[:, :, 3].double() - rk).abs().max() < 1e-5
+    assert torch.equal(vc[:, :, :, 3], qkv[:, H * d:].view(T, G, d))   # raw keys
+
+
+def test_sink_softmax_and_visibility_alone():
+    """ops.paged_attention (one sequence, pages in a shuffled pool) against
+    the oracle's visibility matrix and sink softmax."""
+    from gpustack_amd import ops
+
+    T, H, G, d, dv, window, keep = 45, 4, 2, 6, 5, 9, 3
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn(T, H, d, generator=g)
+    k = torch.randn(T, G, d, generator=g)
+    v = torch.randn(T, G, dv, generator=g)
+    sinks = torch.randn(H, generator=g) * 2
+    blocks = [4, 1, 3]
+    kc, vc = torch.zeros(5, G, 16, d), torch.zeros(5, G, dv, 16)
+    for t in range(T):
+        kc[blocks[t // 16], :, t % 16] = k[t]
+        vc[blocks[t // 16], :, :, t % 16] = v[t]
+    bt = torch.tensor([blocks], dtype=torch.int32)
+    pos = torch.arange(T, dtype=torch.int32)
+    for win, kp, sk in ((window, keep, None), (0, 0, sinks), (window, 0, sinks)):
+        out = torch.zeros(T, H, dv)
+        ops.paged_attention(out, q, kc, vc, bt, torch.zeros(T, dtype=torch.int32),
+                            pos, 0.4, window=win, keep_first=kp, sinks=sk)
+        ok = oracle.visible(T, win, kp)
+        for a in range(H):
+            s = (q[:, a].double() @ k[:, a // 2].double().T) * 0.4
+            s = s.masked_fill(~ok, float("-inf"))
+            ref = oracle.softmax_with_sink(
+                s, None if sk is None else sk[a].double()) @ v[:, a // 2].double()
+            assert (out[:, a].double() - ref).abs().max() < 1e-5
+
 def _one(tmp_path, layers, loop=None, mult=0.7, n=37, seed=0, width=20,
          steps=None, **kw):
     cfg = oracle.make_config(width=width, layers=layers, loop=loop, mult=mult)
